@@ -15,11 +15,13 @@ PAGE_TOKENS = 64  # a sequence's keys and values are stored in pages of this man
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of every position, or of the last ``window`` positions."""
+    """Keys and values of every position, or of the last ``window`` positions. ``value_dim``: the values' width
+    where it differs from the keys' (None: the same)."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None
 
 
 @dataclass(frozen=True)

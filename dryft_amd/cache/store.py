@@ -32,7 +32,7 @@ class KVLine:
     """What an attention-like mixer gets for one cache line."""
 
     k: torch.Tensor           # [pages, kv_heads, 64, head_dim]
-    v: torch.Tensor           # [pages, kv_heads, head_dim, 64]
+    v: torch.Tensor           # [pages, kv_heads, head_dim, 64] (the values' own width where it differs)
     page_table: torch.Tensor  # [slots, max_pages] int32, device
     max_pages: int
     window: int | None
@@ -52,7 +52,7 @@ class KVGroup:
         shape = (len(lines), n_pages, need.num_kv_heads, PAGE_TOKENS, need.head_dim)
         self.k = torch.zeros(shape, dtype=dtype, device=device)
         # values are kept transposed within a page: [.., head_dim, 64], columns in the kernels' own order
-        self.v = torch.zeros(shape[:3] + (need.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
+        self.v = torch.zeros(shape[:3] + (need.value_dim or need.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
         self.table = PageTable(n_slots, n_pages, max_pages, need.window)
         self.table_dev = torch.full((n_slots, max_pages), -1, dtype=torch.int32, device=device)
         self.max_pages = max_pages
@@ -66,7 +66,7 @@ class KVGroup:
         dirty.clear()
 
     def bytes(self) -> int:
-        return 2 * self.k.numel() * self.k.element_size()
+        return (self.k.numel() + self.v.numel()) * self.k.element_size()
 
 
 class StateGroup:
@@ -211,7 +211,8 @@ class CacheStore:
         total = 0.0
         for g in self.kv_groups:
             seen = min(context, g.need.window) if g.need.window else context
-            total += 2.0 * len(g.lines) * g.need.num_kv_heads * g.need.head_dim * g.k.element_size() * seen
+            total += len(g.lines) * g.need.num_kv_heads * (g.need.head_dim + (g.need.value_dim or g.need.head_dim)) * \
+                g.k.element_size() * seen
         for g in self.state_groups:
             total += g.bytes() / self.n_slots
         return total

@@ -43,6 +43,9 @@ class Run:
     layer: int
     cache_line: int
     writes_cache: bool = True
+    # (name of one of the plan's ``stream_parts``, a number of its own): that part acts on the residual stream right
+    # before this run (the start of a pass over a run of layers, for instance)
+    enter: tuple[str, int] | None = None
 
 
 @dataclass(frozen=True)
@@ -55,6 +58,7 @@ class ModelPlan:
     final_norm: PartSpec
     head: PartSpec
     positions: dict[str, PartSpec] = field(default_factory=dict)
+    stream_parts: dict[str, PartSpec] = field(default_factory=dict)   # parts that act between runs (``Run.enter``)
     # Tensors a checkpoint may hold although the model reads them under another name: each maps to the name of
     # the tensor it has to equal when present (a tied head's copy of the embedding).
     optional_tensors: dict[str, str] = field(default_factory=dict)
@@ -66,6 +70,8 @@ class ModelPlan:
         for i, run in enumerate(self.schedule):
             if not 0 <= run.layer < len(self.layers):
                 problems.append(f"schedule[{i}] names layer {run.layer}, plan has {len(self.layers)}")
+            if run.enter is not None and run.enter[0] not in self.stream_parts:
+                problems.append(f"schedule[{i}] enters through {run.enter[0]!r}, which the plan does not have")
             if run.writes_cache:
                 if run.cache_line in writers:
                     problems.append(

@@ -51,3 +51,54 @@ DRYFT_API int dryft_silu_mul(const void* gu, void* y, int n_rows, int inter, int
                        gu_stride);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// A gated linear unit with clamped halves: g = min(gu[:, :I], limit), u = clamp(gu[:, I:], -limit, limit),
+// y = T( g * sigmoid(alpha * g) * (u + 1) ), evaluated in float and rounded once.
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ y, int inter, int64_t gu_stride,
+                                   float limit, float alpha) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= inter) return;
+  const float g = fminf(load_as_float(gu + row * gu_stride + i), limit);
+  const float u = fminf(fmaxf(load_as_float(gu + row * gu_stride + inter + i), -limit), limit);
+  store_from_float(y + row * inter + i, g / (1.f + expf(-alpha * g)) * (u + 1.f));
+}
+
+DRYFT_API int dryft_glu_clamped(const void* gu, void* y, int n_rows, int inter, int64_t gu_stride, float limit,
+                                float alpha, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  dim3 grid(n_rows, (inter + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)y, inter,
+                       gu_stride, limit, alpha);
+  else
+    hipLaunchKernelGGL(glu_clamped_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)y, inter,
+                       gu_stride, limit, alpha);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// An output gate: y = T( a * sigmoid(g) ), a and g rows of `width` values with strides of their own (either
+// may be a run of columns of a wider tensor).
+template <typename T>
+__global__ void sigmoid_gate_kernel(const T* __restrict__ a, int64_t a_stride, const T* __restrict__ g,
+                                    int64_t g_stride, T* __restrict__ y, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const float gate = 1.f / (1.f + expf(-load_as_float(g + row * g_stride + i)));
+  store_from_float(y + row * width + i, load_as_float(a + row * a_stride + i) * gate);
+}
+
+DRYFT_API int dryft_sigmoid_gate(const void* a, int64_t a_stride, const void* g, int64_t g_stride, void* y,
+                                 int n_rows, int width, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  dim3 grid(n_rows, (width + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, block, 0, stream, (const float*)a, a_stride,
+                       (const float*)g, g_stride, (float*)y, width);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)a, a_stride,
+                       (const bf16_t*)g, g_stride, (bf16_t*)y, width);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -8,6 +8,11 @@
 // with lo = 0, or pos - window + 1 for a windowed mixer; query head h reads kv head h / group.
 // Probabilities are rounded to the storage dtype before they weigh the values, as the
 // matrix-core kernels must (attn_decode.py:12-14, 89); with float storage that is the identity.
+//
+// Options that other designs use: a value width v_dim that differs from the key width; a capped score,
+// s <- cap * tanh(s / cap); a sink, one learned number per query head whose exp() joins the softmax's
+// denominator and nothing else (no key, no value; neither scaled nor capped); probabilities kept in
+// float (exact_p), for designs that ask for float attention weights also in bfloat16.
 #include "common.h"
 
 #define ROWS_THREADS 256
@@ -17,7 +22,8 @@ template <typename T>
 __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                                  const int* __restrict__ page_table, int max_pages, const int* __restrict__ row_slot,
                                  const int* __restrict__ row_pos, T* __restrict__ out, int n_heads, int n_kv,
-                                 int head_dim, float scale, int window, int vec) {
+                                 int head_dim, int v_dim, float scale, int window, float softcap,
+                                 const float* __restrict__ sink, int exact_p, int vec) {
   __shared__ float qs[ROWS_MAX_HEAD_DIM];
   __shared__ float ps[ROWS_THREADS];
   __shared__ int pages[ROWS_THREADS / PAGE_TOKENS];
@@ -25,9 +31,9 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
   const int64_t row = blockIdx.x;
   const int head = blockIdx.y, tid = threadIdx.x;
   const int slot = row_slot[row];
-  T* o = out + (row * n_heads + head) * head_dim;
+  T* o = out + (row * n_heads + head) * v_dim;
   if (slot < 0) {
-    if (tid < head_dim) store_from_float(o + tid, 0.f);
+    if (tid < v_dim) store_from_float(o + tid, 0.f);
     return;
   }
   const int pos = row_pos[row];
@@ -60,14 +66,15 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
         for (int i = 0; i < head_dim; ++i) d += qs[i] * load_as_float(kp + i);
       }
       s = d * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m, block_max(s, scratch));  // finite: every chunk holds a key the row sees
     const float alpha = expf(m - m_new);                   // first chunk: exp(-inf) = 0
     const float p = seen ? expf(s - m_new) : 0.f;
     l = l * alpha + block_sum(p, scratch);
-    ps[tid] = rounded_as<T>(p);
+    ps[tid] = exact_p ? p : rounded_as<T>(p);
     __syncthreads();
-    if (tid < head_dim) {
+    if (tid < v_dim) {
       acc *= alpha;
       const int n = min(ROWS_THREADS, pos - c + 1);
       if (vec) {
@@ -77,7 +84,7 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
         for (int pi = 0; pi * PAGE_TOKENS < n; ++pi) {
           const int pg = pages[pi];
           if (pg < 0) continue;
-          const T* vrow = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS;
+          const T* vrow = v_pages + (((int64_t)pg * n_kv + kvh) * v_dim + tid) * PAGE_TOKENS;
           const float* pw = ps + pi * PAGE_TOKENS;
 #pragma unroll
           for (int c8 = 0; c8 < PAGE_TOKENS / 8; ++c8) {
@@ -92,31 +99,41 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
         for (int jj = 0; jj < n; ++jj) {
           const int pg = pages[jj / PAGE_TOKENS];
           if (pg < 0) continue;
-          const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * head_dim + tid) * PAGE_TOKENS + value_column(jj % PAGE_TOKENS);
+          const T* vp = v_pages + (((int64_t)pg * n_kv + kvh) * v_dim + tid) * PAGE_TOKENS + value_column(jj % PAGE_TOKENS);
           acc += ps[jj] * load_as_float(vp);
         }
       }
     }
     m = m_new;
   }
-  if (tid < head_dim) store_from_float(o + tid, acc / l);
+  if (sink != nullptr) {                                   // the sink counts once in the denominator
+    const float sk = sink[head];
+    if (sk > m) {
+      const float a = expf(m - sk);
+      l = l * a + 1.f;
+      acc *= a;
+    } else {
+      l += expf(sk - m);
+    }
+  }
+  if (tid < v_dim) store_from_float(o + tid, acc / l);
 }
 
 DRYFT_API int dryft_attn_rows(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                               int max_pages, const int* row_slot, const int* row_pos, void* out, int n_rows,
-                              int n_heads, int n_kv, int head_dim, float scale, int window, int is_f32,
-                              hipStream_t stream) {
+                              int n_heads, int n_kv, int head_dim, int v_dim, float scale, int window, float softcap,
+                              const float* sink, int exact_p, int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (head_dim > ROWS_MAX_HEAD_DIM || n_kv <= 0 || n_heads % n_kv) return -1;
+  if (head_dim > ROWS_MAX_HEAD_DIM || v_dim <= 0 || v_dim > ROWS_THREADS || n_kv <= 0 || n_heads % n_kv) return -1;
   dim3 grid(n_rows, n_heads), block(ROWS_THREADS);
-  const int vec = head_dim % 8 == 0 && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
+  const int vec = head_dim % 8 == 0 && v_dim % 8 == 0 && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
   if (is_f32)
     hipLaunchKernelGGL(attn_rows_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_pages,
                        (const float*)v_pages, page_table, max_pages, row_slot, row_pos, (float*)out, n_heads, n_kv,
-                       head_dim, scale, window, vec);
+                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec);
   else
     hipLaunchKernelGGL(attn_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
                        (const bf16_t*)v_pages, page_table, max_pages, row_slot, row_pos, (bf16_t*)out, n_heads, n_kv,
-                       head_dim, scale, window, vec);
+                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec);
   return DRYFT_LAUNCH_CHECK();
 }

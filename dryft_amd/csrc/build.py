@@ -25,7 +25,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-MODULES = ("batch", "embed", "norm", "activation", "rope_kv", "attn_rows", "attn_mfma", "gemm", "sampling")
+MODULES = ("batch", "embed", "norm", "activation", "rope_kv", "attn_rows", "attn_mfma", "gemm", "sampling", "mlstm",
+           "rglru")
 _HEADERS = ("common.h",)                       # every library includes these
 _OWN_HEADERS = {"sampling": ("sampling.h",)}    # and some a header of their own
 

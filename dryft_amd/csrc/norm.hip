@@ -177,3 +177,80 @@ DRYFT_API int dryft_add_rows(const void* a, const void* b, void* out, int64_t n,
                        (bf16_t*)out, n);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// The norms of a float32 residual stream, for layers that norm a branch's output before it is added
+// and norm the stream again for the next branch. One launch does, per row,
+//
+//   d      = sum_p delta[p]                                     (the branch's output; T, or float partial sums)
+//   x_new  = x + d * rsqrt(mean(d^2) + eps) * wb + extra + vec   (each term optional; without wb, d is added as it is)
+//   y      = T( x_new * rsqrt(mean(x_new^2) + eps) * w )         (optional)
+//
+// with x given as float32, in the activation dtype (the embedding's output, which starts a stream) or
+// not at all, `extra` a row tensor in the activation dtype and `vec` one vector for every row. All of it
+// is float arithmetic; only y is rounded, once. The row is held in LDS between the passes (dynamic
+// shared memory of `width` floats), and a thread touches the same elements in every pass.
+template <typename T, typename D>
+__global__ __launch_bounds__(256) void stream_norm_kernel(const void* __restrict__ x_in, int x_kind,
+                                                          const D* __restrict__ delta, int n_partials,
+                                                          int64_t partial_stride, const void* __restrict__ wb,
+                                                          int wb_f32, const T* __restrict__ extra,
+                                                          const void* __restrict__ vec, int vec_f32,
+                                                          const void* __restrict__ w, int w_f32,
+                                                          float* __restrict__ x_out, T* __restrict__ y, int width,
+                                                          float eps) {
+  extern __shared__ float held[];
+  __shared__ float scratch[16];
+  const int64_t base = (int64_t)blockIdx.x * width;
+  float inv_d = 1.f;
+  if (n_partials > 0) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      float d = 0.f;
+      for (int p = 0; p < n_partials; ++p) d += load_as_float(delta + p * partial_stride + base + i);
+      held[i] = d;
+      ss += d * d;
+    }
+    if (wb != nullptr) inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = 0.f;
+    if (x_kind == 2) v = ((const float*)x_in)[base + i];
+    else if (x_kind == 1) v = load_as_float((const T*)x_in + base + i);
+    if (n_partials > 0) v += wb != nullptr ? held[i] * inv_d * load_vector(wb, i, wb_f32) : held[i];
+    if (extra != nullptr) v += load_as_float(extra + base + i);
+    if (vec != nullptr) v += load_vector(vec, i, vec_f32);
+    held[i] = v;
+    if (x_out != nullptr) x_out[base + i] = v;
+    ss += v * v;
+  }
+  if (y == nullptr) return;
+  const float inv = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    store_from_float(y + base + i, held[i] * inv * load_vector(w, i, w_f32));
+}
+
+#define STREAM_NORM_MAX_WIDTH 16384   // 64 KiB of LDS a row
+
+// x_kind: 0 = no stream yet, 1 = the stream in the activation dtype, 2 = float32.
+// delta_kind: 0 = none, 1 = activation dtype, 2 = float partial sums.
+DRYFT_API int dryft_stream_norm(const void* x_in, int x_kind, const void* delta, int delta_kind, int n_partials,
+                                int64_t partial_stride, const void* wb, int wb_f32, const void* extra,
+                                const void* vec, int vec_f32, const void* w, int w_f32, float* x_out, void* y,
+                                int n_rows, int width, float eps, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0 || width > STREAM_NORM_MAX_WIDTH || (y != nullptr && w == nullptr)) return -1;
+  if (delta_kind == 0) n_partials = 0;
+  dim3 grid(n_rows), block(256);
+  const size_t lds = (size_t)width * sizeof(float);
+#define SN(TT, DD)                                                                                                   \
+  hipLaunchKernelGGL((stream_norm_kernel<TT, DD>), grid, block, lds, stream, x_in, x_kind, (const DD*)delta,        \
+                     n_partials, partial_stride, wb, wb_f32, (const TT*)extra, vec, vec_f32, w, w_f32, x_out,       \
+                     (TT*)y, width, eps)
+  if (is_f32) SN(float, float);
+  else if (delta_kind == 2) SN(bf16_t, float);
+  else SN(bf16_t, bf16_t);
+#undef SN
+  return DRYFT_LAUNCH_CHECK();
+}

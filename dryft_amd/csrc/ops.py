@@ -22,14 +22,25 @@ _SIGNATURES = {
               "dryft_tile_prefix": [_P, _P, _I, _I, _P, _P]},
     "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _I, _P]},
     "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
-             "dryft_add_rows": [_P, _P, _P, _L, _I, _P]},
-    "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P]},
+             "dryft_add_rows": [_P, _P, _P, _L, _I, _P],
+             "dryft_stream_norm": [_P, _I, _P, _I, _I, _L, _P, _I, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I, _P]},
+    "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P],
+                   "dryft_glu_clamped": [_P, _P, _I, _I, _L, _F, _F, _I, _P],
+                   "dryft_sigmoid_gate": [_P, _L, _P, _L, _P, _I, _I, _I, _P]},
+    "mlstm": {"dryft_mlstm_steps": [_P, _L, _I, _I, _I, _P, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F,
+                                    _I, _I, _P],
+              "dryft_mlstm_out": [_P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
+    "rglru": {"dryft_rglru_gates": [_P, _L, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _P, _P, _I, _I,
+                                    _I, _I, _P],
+              "dryft_rglru_scan": [_P, _P, _L, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]},
     "rope_kv": {"dryft_qk_norm_rope_kv": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                           _I, _I, _I, _I, _I, _P],
+                "dryft_rope_pairs_kv": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                        _I, _I, _P],
                 "dryft_rows_to_cache_takes": [_I, _I, _I, _I],
                 "dryft_rows_to_cache_parts": [_P, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                               _I, _I, _I, _P]},
-    "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P]},
+    "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_causal_takes_projection": [_I, _I],
                   "dryft_attn_causal_projected_bf16": [_P, _L, _P, _I, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I,
@@ -212,7 +223,92 @@ def add_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tenso
     return out
 
 
+def stream_norm(x, delta, post_weight, extra, vec, weight, eps: float, x_out, y, act: torch.dtype) -> None:
+    """The norms of a float32 residual stream in one launch, per row:
+    ``d = delta`` (a tensor in the activation dtype, or ``[n, rows, width]`` float32 partial sums as ``(data, n)``);
+    ``x_out = x + rmsnorm(d) * post_weight + extra + vec`` (each term optional; without ``post_weight`` ``d`` is added
+    as it is); ``y = rmsnorm(x_out) * weight`` in the activation dtype (optional). ``x`` is float32, or in the
+    activation dtype ``act`` (a stream that starts), or None; ``x_out`` is float32 (may be ``x`` itself) or None."""
+    ref = y if y is not None else (x_out if x_out is not None else x)
+    rows, width = ref.shape
+    x_kind = 0
+    if x is not None:
+        _gpu(x, "x")
+        if not (x.shape == (rows, width) and x.is_contiguous()):
+            raise KernelError("stream_norm: x must be contiguous [rows, width]")
+        x_kind = 1 if (x.dtype == act and x is not x_out) else 2
+    n_partials, kind, stride = 0, 0, 0
+    if delta is not None:
+        data, n_partials = delta if isinstance(delta, tuple) else (delta, 1)
+        _gpu(data, "delta")
+        if isinstance(delta, tuple):
+            if not (data.dtype == torch.float32 and data.dim() == 3 and data.shape[1:] == (rows, width) and
+                    data.is_contiguous() and data.shape[0] >= n_partials >= 1):
+                raise KernelError("stream_norm: partial sums must be contiguous float32 [n, rows, width]")
+            kind, stride = 2, rows * width
+        else:
+            if not (data.shape == (rows, width) and data.is_contiguous()):
+                raise KernelError("stream_norm: delta must be contiguous [rows, width]")
+            kind = 1
+        delta = data
+    for name, t in (("post_weight", post_weight), ("vec", vec), ("weight", weight)):
+        if t is not None:
+            _gpu(t, name)
+            _float_flag(t, name)
+            if not (t.shape == (width,) and t.is_contiguous()):
+                raise KernelError(f"stream_norm: {name} must be [{width}]")
+    is_f32 = 1 if act == torch.float32 else 0
+    if kind == 1 and delta.dtype != act or x_kind == 2 and x.dtype != torch.float32:
+        raise KernelError("stream_norm: delta must be in the activation dtype, the stream in it or in float32")
+    if extra is not None:
+        _gpu(extra, "extra", act)
+        if not (extra.shape == (rows, width) and extra.is_contiguous()):
+            raise KernelError("stream_norm: extra must be contiguous [rows, width]")
+    if x_out is not None:
+        _gpu(x_out, "x_out", torch.float32)
+        if not (x_out.shape == (rows, width) and x_out.is_contiguous()):
+            raise KernelError("stream_norm: x_out must be contiguous float32 [rows, width]")
+    if y is not None:
+        _gpu(y, "y", act)
+        if not (y.is_contiguous() and weight is not None):
+            raise KernelError("stream_norm: y contiguous, and a weight for it")
+    flag = lambda t: 0 if t is None else _float_flag(t, "vector")      # noqa: E731
+    _check(_fn("norm", "dryft_stream_norm")(
+        _ptr(x), x_kind, _ptr(delta), kind, n_partials, stride, _ptr(post_weight), flag(post_weight), _ptr(extra),
+        _ptr(vec), flag(vec), _ptr(weight), flag(weight), _ptr(x_out), _ptr(y), rows, width, float(eps), is_f32,
+        _stream()), "stream_norm")
+
+
 # -------------------------------------------------------------------------------------- activation
+def glu_clamped(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """``out = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(gate_up[:, :I], limit)`` and
+    ``u = clamp(gate_up[:, I:], -limit, limit)``."""
+    _gpu(gate_up, "gate_up")
+    _gpu(out, "out", gate_up.dtype)
+    rows, two = gate_up.shape
+    inter = two // 2
+    if not (two == 2 * inter and gate_up.stride(1) == 1 and out.shape == (rows, inter) and out.is_contiguous()):
+        raise KernelError("glu_clamped: gate_up [rows, 2I] with unit column stride, out contiguous [rows, I]")
+    _check(_fn("activation", "dryft_glu_clamped")(_ptr(gate_up), _ptr(out), rows, inter, gate_up.stride(0), float(limit),
+                                                  float(alpha), _float_flag(gate_up, "gate_up"), _stream()),
+           "glu_clamped")
+    return out
+
+
+def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out = a * sigmoid(gate)``; ``a`` and ``gate`` are ``[rows, width]`` and may be column runs of wider tensors."""
+    _gpu(a, "a")
+    _gpu(gate, "gate", a.dtype)
+    _gpu(out, "out", a.dtype)
+    rows, width = a.shape
+    if not (gate.shape == a.shape and a.stride(1) == 1 and gate.stride(1) == 1 and out.shape == a.shape and
+            out.is_contiguous()):
+        raise KernelError("sigmoid_gate: a and gate [rows, width] with unit column stride, out contiguous")
+    _check(_fn("activation", "dryft_sigmoid_gate")(_ptr(a), a.stride(0), _ptr(gate), gate.stride(0), _ptr(out), rows,
+                                                   width, _float_flag(a, "a"), _stream()), "sigmoid_gate")
+    return out
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _gpu(gate_up, "gate_up")
     _gpu(out, "out", gate_up.dtype)
@@ -328,11 +424,13 @@ def rows_to_cache_from_partials(parts: torch.Tensor, q_weight, k_weight, eps: fl
         _ptr(page_table), page_table.shape[1], rows, n_heads, n_kv, head_dim, _stream()), "rows_to_cache_parts")
 
 
-def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype) -> None:
-    for name, t in (("k_pages", k_pages), ("v_pages", v_pages)):
+def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype, v_dim: int | None = None) -> None:
+    for name, t, d in (("k_pages", k_pages, head_dim), ("v_pages", v_pages, head_dim if v_dim is None else v_dim)):
         _gpu(t, name, dtype)
-        if not (t.dim() == 4 and t.shape[1] == n_kv and t.shape[2] * t.shape[3] == 64 * head_dim and t.is_contiguous()):
-            raise KernelError(f"{name}: must be contiguous [pages, {n_kv}, 64, {head_dim}], got {tuple(t.shape)}")
+        if not (t.dim() == 4 and t.shape[1] == n_kv and t.shape[2] * t.shape[3] == 64 * d and t.is_contiguous()):
+            raise KernelError(f"{name}: must be contiguous [pages, {n_kv}, 64, {d}], got {tuple(t.shape)}")
+    if k_pages.shape[0] != v_pages.shape[0]:
+        raise KernelError("k_pages and v_pages: different numbers of pages")
     _gpu(page_table, "page_table", torch.int32)
     if not (page_table.dim() == 2 and page_table.is_contiguous()):
         raise KernelError("page_table: must be contiguous [slots, pages]")
@@ -340,16 +438,25 @@ def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype) 
 
 # --------------------------------------------------------------------------------------- attention
 def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: int, n_kv: int, head_dim: int,
-              scale: float, window: int) -> None:
+              scale: float, window: int, *, v_dim: int | None = None, softcap: float = 0.0, sink=None,
+              exact_p: bool = False) -> None:
+    """``v_dim``: the values' width where it differs from the keys'; ``softcap`` > 0: scores become
+    ``cap * tanh(s / cap)``; ``sink``: float32 ``[heads]`` whose exp() joins each head's denominator; ``exact_p``:
+    the probabilities weigh the values unrounded."""
     _gpu(q, "q")
     is_f32 = _float_flag(q, "q")
+    v_dim = head_dim if v_dim is None else int(v_dim)
     rows = q.numel() // (n_heads * head_dim)
     if not (q.is_contiguous() and q.numel() == rows * n_heads * head_dim):
         raise KernelError("attn_rows: q must be [rows, heads, head_dim]")
     _gpu(out, "out", q.dtype)
-    if not (out.is_contiguous() and out.numel() == q.numel()):
-        raise KernelError("attn_rows: out like q")
-    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, q.dtype)
+    if not (out.is_contiguous() and out.numel() == rows * n_heads * v_dim):
+        raise KernelError("attn_rows: out must be [rows, heads, v_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, q.dtype, v_dim)
+    if sink is not None:
+        _gpu(sink, "sink", torch.float32)
+        if not (sink.is_contiguous() and sink.numel() == n_heads):
+            raise KernelError(f"sink: needs {n_heads} entries")
     for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
         _gpu(t, name, torch.int32)
         if not (t.numel() >= rows):
@@ -358,7 +465,8 @@ def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: 
         raise KernelError("attn_rows: too many heads")
     _check(_fn("attn_rows", "dryft_attn_rows")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(row_slot), _ptr(row_pos),
-        _ptr(out), rows, n_heads, n_kv, head_dim, float(scale), int(window), is_f32, _stream()), "attn_rows")
+        _ptr(out), rows, n_heads, n_kv, head_dim, v_dim, float(scale), int(window), float(softcap), _ptr(sink),
+        int(bool(exact_p)), is_f32, _stream()), "attn_rows")
 
 
 ATTN_ROW_TILE = 64      # rows of a sequence that one workgroup of the prompt-attention kernels takes (``tile_cu``)
@@ -895,3 +1003,186 @@ def sample_rows(logits: torch.Tensor, temperature: float, uniforms: torch.Tensor
                                                 _ptr(uniforms), _ptr(out), chunks, _ptr(chunk_max), _ptr(chunk_sum),
                                                 _stream()), "sample_rows")
     return out
+
+
+# --------------------------------------------------------------------------------- rotary over neighbouring pairs
+def rope_pairs_kv(proj, q_col: int, k_col: int, v_col: int, cos, sin, rot: int, row_slot, row_pos, q_out, k_pages,
+                  v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int, head_dim: int, v_dim: int) -> None:
+    """Rotates the q and k heads of a fused projection pair by pair ``(2i, 2i + 1)`` over their first ``rot`` features
+    with float32 tables ``[positions, rot / 2]``, writes the queries to ``q_out [rows, heads, head_dim]`` and, when
+    ``write_kv``, the keys and the (unrotated) values of width ``v_dim`` to their pages."""
+    _gpu(proj, "proj")
+    is_f32 = _float_flag(proj, "proj")
+    rows = proj.shape[0]
+    if not (proj.dim() == 2 and proj.stride(1) == 1):
+        raise KernelError("rope_pairs_kv: proj must be [rows, columns] with unit column stride")
+    ends = (q_col + n_heads * head_dim, k_col + n_kv * head_dim, v_col + n_kv * v_dim)
+    if min(q_col, k_col, v_col) < 0 or max(ends) > proj.shape[1]:
+        raise KernelError("rope_pairs_kv: q, k or v lie outside the projection's columns")
+    if rot % 2 or not 0 <= rot <= head_dim:
+        raise KernelError(f"rope_pairs_kv: the rotated width must be even and at most {head_dim}, got {rot}")
+    if rot:
+        for name, t in (("cos", cos), ("sin", sin)):
+            _gpu(t, name, torch.float32)
+            if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+                raise KernelError(f"{name}: must be contiguous float32 [positions, {rot // 2}]")
+    _gpu(q_out, "q_out", proj.dtype)
+    if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim):
+        raise KernelError("rope_pairs_kv: q_out must be [rows, heads, head_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, proj.dtype, v_dim)
+    for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        if not (t.numel() >= rows):
+            raise KernelError(f"{name}: needs {rows} entries")
+    _check(_fn("rope_kv", "dryft_rope_pairs_kv")(
+        _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(cos), _ptr(sin), rot, _ptr(row_slot), _ptr(row_pos),
+        _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], int(bool(write_kv)), rows,
+        n_heads, n_kv, head_dim, v_dim, is_f32, _stream()), "rope_pairs_kv")
+
+
+# ------------------------------------------------------------------------------------------ recurrent mixers
+def _f32_vector(t, name: str, n: int) -> None:
+    _gpu(t, name, torch.float32)
+    if not (t.is_contiguous() and t.numel() == n):
+        raise KernelError(f"{name}: needs {n} contiguous float32 entries, has {tuple(t.shape)}")
+
+
+def _seq_facts(seq_slot, cu_rows, q_len, n_seqs: int) -> None:
+    for name, t, n in (("seq_slot", seq_slot, n_seqs), ("cu_rows", cu_rows, n_seqs + 1), ("q_len", q_len, n_seqs)):
+        _gpu(t, name, torch.int32)
+        if not (t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"{name}: needs {n} contiguous entries")
+
+
+MLSTM_MAX_DIM = 256
+
+
+def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f, cap: float, seq_slot, cu_rows, q_len,
+                n_seqs: int, state_s, state_n, state_m, o_raw, n_heads: int, dim: int, v_dim: int, q_scale: float,
+                write_state: bool) -> None:
+    """The matrix-memory recurrence over each sequence's rows of the step, in order; ``o_raw`` (float32
+    ``[rows, heads, v_dim]``) receives each token's read-out divided by its normaliser. ``gates`` are the float32
+    projections ``[rows, 2 * heads]`` (input gates, then forget gates) before bias, cap and log-sigmoid. The states
+    ``[slots, heads, dim, v_dim]``, ``[slots, heads, dim]`` and ``[slots, heads]`` are float32."""
+    _gpu(proj, "proj")
+    is_f32 = _float_flag(proj, "proj")
+    rows = proj.shape[0]
+    if not (proj.dim() == 2 and proj.stride(1) == 1):
+        raise KernelError("mlstm_steps: proj must be [rows, columns] with unit column stride")
+    if min(q_col, k_col, v_col) < 0 or max(q_col + n_heads * dim, k_col + n_heads * dim,
+                                           v_col + n_heads * v_dim) > proj.shape[1]:
+        raise KernelError("mlstm_steps: q, k or v lie outside the projection's columns")
+    if not 0 < dim <= MLSTM_MAX_DIM:
+        raise KernelError(f"mlstm_steps: key width must lie in 1..{MLSTM_MAX_DIM}, got {dim}")
+    _gpu(gates, "gates", torch.float32)
+    if not (gates.shape == (rows, 2 * n_heads) and gates.is_contiguous()):
+        raise KernelError(f"mlstm_steps: gates must be contiguous float32 [{rows}, {2 * n_heads}]")
+    _f32_vector(bias_i, "bias_i", n_heads)
+    _f32_vector(bias_f, "bias_f", n_heads)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    slots = state_m.shape[0]
+    for name, t, shape in (("state_s", state_s, (slots, n_heads, dim, v_dim)), ("state_n", state_n, (slots, n_heads, dim)),
+                           ("state_m", state_m, (slots, n_heads))):
+        _gpu(t, name, torch.float32)
+        if not (tuple(t.shape) == shape and t.is_contiguous()):
+            raise KernelError(f"{name}: must be contiguous float32 {shape}, got {tuple(t.shape)}")
+    _gpu(o_raw, "o_raw", torch.float32)
+    if not (o_raw.is_contiguous() and o_raw.numel() == rows * n_heads * v_dim):
+        raise KernelError("mlstm_steps: o_raw must be float32 [rows, heads, v_dim]")
+    _check(_fn("mlstm", "dryft_mlstm_steps")(
+        _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),
+        _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs, _ptr(state_s), _ptr(state_n), _ptr(state_m), _ptr(o_raw),
+        n_heads, dim, v_dim, float(q_scale), int(bool(write_state)), is_f32, _stream()), "mlstm_steps")
+
+
+def mlstm_out(o_raw, proj, g_col: int, weight, row_slot, out, n_heads: int, v_dim: int, eps: float) -> None:
+    """``out = o_raw / rms_per_head(o_raw) * weight * sigmoid(proj[:, g_col:...])`` in the activation dtype."""
+    _gpu(proj, "proj")
+    rows = proj.shape[0]
+    _gpu(o_raw, "o_raw", torch.float32)
+    _gpu(out, "out", proj.dtype)
+    if not (o_raw.is_contiguous() and o_raw.numel() == rows * n_heads * v_dim and out.is_contiguous() and
+            out.numel() == o_raw.numel()):
+        raise KernelError("mlstm_out: o_raw and out must hold [rows, heads, v_dim]")
+    if not (proj.stride(1) == 1 and 0 <= g_col and g_col + n_heads * v_dim <= proj.shape[1]):
+        raise KernelError("mlstm_out: the gate lies outside the projection's columns")
+    _f32_vector(weight, "weight", n_heads * v_dim)
+    _gpu(row_slot, "row_slot", torch.int32)
+    _check(_fn("mlstm", "dryft_mlstm_out")(_ptr(o_raw), _ptr(proj), proj.stride(0), g_col, _ptr(weight), _ptr(row_slot),
+                                           _ptr(out), rows, n_heads, v_dim, float(eps),
+                                           _float_flag(proj, "proj"), _stream()), "mlstm_out")
+
+
+RGLRU_MAX_TAPS = 16
+
+
+def rglru_gates(proj, x_col: int, x_bias, conv_w, conv_b, taps: int, gate_a, gate_a_bias, gate_i, gate_i_bias, lam,
+                decay_scale: float, row_slot, row_seq, row_pos, seq_start, tail, coef, width: int, blocks: int) -> None:
+    """Per row and channel the recurrence's two coefficients, ``coef[row, 0] = a`` and
+    ``coef[row, 1] = sqrt(1 - a^2) * i * u``, from the convolution of the recurrent branch (columns ``x_col..`` of
+    ``proj`` plus ``x_bias``; inputs before the step come from ``tail [slots, taps - 1, width]``) and the
+    block-diagonal gates ``gate_a``, ``gate_i`` ``[blocks, width / blocks, width / blocks]``."""
+    _gpu(proj, "proj")
+    is_f32 = _float_flag(proj, "proj")
+    rows = proj.shape[0]
+    if not (proj.dim() == 2 and proj.stride(1) == 1 and 0 <= x_col and x_col + width <= proj.shape[1]):
+        raise KernelError("rglru_gates: the branch lies outside the projection's columns")
+    if blocks <= 0 or width % blocks or not 1 <= taps <= RGLRU_MAX_TAPS:
+        raise KernelError(f"rglru_gates: {width} channels in {blocks} blocks, {taps} taps")
+    bs = width // blocks
+    for name, t in (("gate_a", gate_a), ("gate_i", gate_i)):
+        _gpu(t, name, proj.dtype)
+        if not (tuple(t.shape) == (blocks, bs, bs) and t.is_contiguous()):
+            raise KernelError(f"{name}: must be contiguous [{blocks}, {bs}, {bs}]")
+    for name, t in (("x_bias", x_bias), ("conv_b", conv_b), ("gate_a_bias", gate_a_bias), ("gate_i_bias", gate_i_bias),
+                    ("lam", lam)):
+        _f32_vector(t, name, width)
+    _f32_vector(conv_w, "conv_w", width * taps)
+    if taps > 1:
+        _gpu(tail, "tail", torch.float32)
+        if not (tail.dim() == 3 and tuple(tail.shape[1:]) == (taps - 1, width) and tail.is_contiguous()):
+            raise KernelError(f"tail: must be contiguous float32 [slots, {taps - 1}, {width}]")
+    for name, t in (("row_slot", row_slot), ("row_seq", row_seq), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        if not (t.numel() >= rows):
+            raise KernelError(f"{name}: needs {rows} entries")
+    _gpu(seq_start, "seq_start", torch.int32)
+    _gpu(coef, "coef", torch.float32)
+    if not (tuple(coef.shape) == (rows, 2, width) and coef.is_contiguous()):
+        raise KernelError(f"coef: must be contiguous float32 [{rows}, 2, {width}]")
+    _check(_fn("rglru", "dryft_rglru_gates")(
+        _ptr(proj), proj.stride(0), x_col, _ptr(x_bias), _ptr(conv_w), _ptr(conv_b), taps, _ptr(gate_a),
+        _ptr(gate_a_bias), _ptr(gate_i), _ptr(gate_i_bias), _ptr(lam), float(decay_scale), _ptr(row_slot), _ptr(row_seq),
+        _ptr(row_pos), _ptr(seq_start), _ptr(tail) if taps > 1 else 0, _ptr(coef), rows, width, blocks, is_f32,
+        _stream()), "rglru_gates")
+
+
+def rglru_scan(coef, proj, x_col: int, y_col: int, x_bias, y_bias, taps: int, seq_slot, cu_rows, q_len, row_slot,
+               n_seqs: int, state, tail, out, width: int, write_state: bool) -> None:
+    """Walks each sequence's rows in order: ``S = a S + b``, ``out = S * gelu_tanh(y + y_bias)``; leaves ``S`` in
+    ``state [slots, width]`` and the sequence's last ``taps - 1`` inputs in ``tail``."""
+    _gpu(proj, "proj")
+    rows = proj.shape[0]
+    _gpu(coef, "coef", torch.float32)
+    if not (tuple(coef.shape) == (rows, 2, width) and coef.is_contiguous()):
+        raise KernelError(f"coef: must be contiguous float32 [{rows}, 2, {width}]")
+    if not (proj.stride(1) == 1 and min(x_col, y_col) >= 0 and max(x_col, y_col) + width <= proj.shape[1]):
+        raise KernelError("rglru_scan: a branch lies outside the projection's columns")
+    _f32_vector(x_bias, "x_bias", width)
+    _f32_vector(y_bias, "y_bias", width)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(row_slot, "row_slot", torch.int32)
+    _gpu(state, "state", torch.float32)
+    if not (state.dim() == 2 and state.shape[1] == width and state.is_contiguous()):
+        raise KernelError(f"state: must be contiguous float32 [slots, {width}]")
+    if taps > 1:
+        _gpu(tail, "tail", torch.float32)
+        if not (tuple(tail.shape) == (state.shape[0], taps - 1, width) and tail.is_contiguous()):
+            raise KernelError(f"tail: must be contiguous float32 [slots, {taps - 1}, {width}]")
+    _gpu(out, "out", proj.dtype)
+    if not (tuple(out.shape) == (rows, width) and out.is_contiguous()):
+        raise KernelError(f"out: must be contiguous [{rows}, {width}]")
+    _check(_fn("rglru", "dryft_rglru_scan")(
+        _ptr(coef), _ptr(proj), proj.stride(0), x_col, y_col, _ptr(x_bias), _ptr(y_bias), taps, _ptr(seq_slot),
+        _ptr(cu_rows), _ptr(q_len), _ptr(row_slot), n_seqs, _ptr(state), _ptr(tail) if taps > 1 else 0, _ptr(out), rows,
+        width, int(bool(write_state)), _float_flag(proj, "proj"), _stream()), "rglru_scan")

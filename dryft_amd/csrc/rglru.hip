@@ -1,0 +1,166 @@
+// A real-gated linear recurrent unit behind a short causal convolution (the recurrent block of Griffin),
+// per sequence and channel. With x the recurrent branch's projection plus its bias, per channel c:
+//
+//   u_t = cb[c] + sum_j cw[c, j] x_(t - (taps - 1 - j))            (zeros before the sequence starts)
+//   r = sigmoid(A_b u_b + ab),  i = sigmoid(I_b u_b + ib)          (u cut into equal blocks b, A_b and I_b square)
+//   log a = -c_a * r * softplus(lam),  a = exp(log a)
+//   S_t = a S_(t-1) + sqrt(1 - a^2) * i * u_t,     out_t = T( S_t * gelu_tanh(y_t + yb) )
+//
+// with y the other branch's projection. S and the last taps - 1 values of x live in float32 in the state
+// store (zero when a sequence starts); everything above is float arithmetic and only out is rounded.
+// Two kernels: the gates of every row at once (a workgroup takes a few rows of one block, so that each
+// gate weight it reads serves all of them), then the walk over a sequence's rows, one thread a channel,
+// which also leaves the state for the next step.
+#include "common.h"
+
+#define RG_ROWS 8               // rows a gates workgroup takes
+#define RG_MAX_TAPS 16
+
+__device__ __forceinline__ float gelu_tanh(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float soft_plus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+
+// coef: float32 [rows, 2, width]: a, then sqrt(1 - a^2) * i * u.
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_gates_kernel(
+    const T* __restrict__ proj, int64_t proj_stride, int x_col, const float* __restrict__ x_bias,
+    const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps, const T* __restrict__ gate_a,
+    const float* __restrict__ gate_a_bias, const T* __restrict__ gate_i, const float* __restrict__ gate_i_bias,
+    const float* __restrict__ lam, float decay_scale, const int* __restrict__ row_slot,
+    const int* __restrict__ row_seq, const int* __restrict__ row_pos, const int* __restrict__ seq_start,
+    const float* __restrict__ tail, float* __restrict__ coef, int n_rows, int width, int block_size) {
+  extern __shared__ float u_s[];                                // [RG_ROWS][block_size]
+  const int r0 = blockIdx.x * RG_ROWS, b = blockIdx.y;
+  const int rows = min(RG_ROWS, n_rows - r0);
+  for (int e = threadIdx.x; e < rows * block_size; e += blockDim.x) {
+    const int rr = e / block_size, c = e % block_size, ch = b * block_size + c;
+    const int64_t row = r0 + rr;
+    const int slot = row_slot[row];
+    float u = 0.f;
+    if (slot >= 0) {
+      const int pos = row_pos[row], start = seq_start[row_seq[row]];
+      u = conv_b[ch];
+      for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j, p = pos - back;
+        float x;
+        if (p >= start) x = load_as_float(proj + (row - back) * proj_stride + x_col + ch) + x_bias[ch];
+        else x = tail[((int64_t)slot * (taps - 1) + (taps - 1 - start + p)) * width + ch];   // zeros before the start
+        u += conv_w[ch * taps + j] * x;
+      }
+    }
+    u_s[e] = u;
+  }
+  __syncthreads();
+  for (int o = threadIdx.x; o < block_size; o += blockDim.x) {
+    const int ch = b * block_size + o;
+    const T* wa = gate_a + ((int64_t)b * block_size + o) * block_size;
+    const T* wi = gate_i + ((int64_t)b * block_size + o) * block_size;
+    float acc_a[RG_ROWS], acc_i[RG_ROWS];
+#pragma unroll
+    for (int rr = 0; rr < RG_ROWS; ++rr) acc_a[rr] = acc_i[rr] = 0.f;
+    for (int k = 0; k < block_size; ++k) {
+      const float a = load_as_float(wa + k), i = load_as_float(wi + k);
+#pragma unroll
+      for (int rr = 0; rr < RG_ROWS; ++rr) {
+        const float u = rr < rows ? u_s[rr * block_size + k] : 0.f;
+        acc_a[rr] += a * u;
+        acc_i[rr] += i * u;
+      }
+    }
+    const float rate = decay_scale * soft_plus(lam[ch]);
+#pragma unroll
+    for (int rr = 0; rr < RG_ROWS; ++rr) {
+      if (rr >= rows || row_slot[r0 + rr] < 0) continue;
+      const float r = 1.f / (1.f + expf(-(acc_a[rr] + gate_a_bias[ch])));
+      const float i = 1.f / (1.f + expf(-(acc_i[rr] + gate_i_bias[ch])));
+      const float log_a = -rate * r;
+      float* dst = coef + (int64_t)(r0 + rr) * 2 * width;
+      dst[ch] = expf(log_a);
+      dst[width + ch] = sqrtf(-expm1f(2.f * log_a)) * i * u_s[rr * block_size + o];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(
+    const float* __restrict__ coef, const T* __restrict__ proj, int64_t proj_stride, int x_col, int y_col,
+    const float* __restrict__ x_bias, const float* __restrict__ y_bias, int taps, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_rows, const int* __restrict__ q_len, const int* __restrict__ row_slot,
+    float* __restrict__ state, float* __restrict__ tail, T* __restrict__ out, int n_rows, int width, int write_state) {
+  const int seq = blockIdx.x, ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= width) return;
+  const int slot = seq_slot[seq];
+  const int row0 = cu_rows[seq], n_tok = q_len[seq];
+  if (slot < 0) {                                               // the rows of a sequence that sits out hold zeros
+    for (int t = 0; t < n_tok; ++t) store_from_float(out + (int64_t)(row0 + t) * width + ch, 0.f);
+    return;
+  }
+  float S = state[(int64_t)slot * width + ch];
+  const float yb = y_bias[ch];
+  for (int t = 0; t < n_tok; ++t) {
+    const int64_t row = row0 + t;
+    const float* c = coef + row * 2 * width;
+    S = c[ch] * S + c[width + ch];
+    const float y = gelu_tanh(load_as_float(proj + row * proj_stride + y_col + ch) + yb);
+    store_from_float(out + row * width + ch, S * y);
+  }
+  if (!write_state) return;
+  state[(int64_t)slot * width + ch] = S;
+  // the convolution's memory: the last taps - 1 inputs of the sequence, oldest first
+  const int keep = taps - 1;
+  float old[RG_MAX_TAPS];
+  float* tl = tail + (int64_t)slot * keep * width + ch;
+  for (int j = 0; j < keep; ++j) old[j] = tl[(int64_t)j * width];
+  for (int j = 0; j < keep; ++j) {
+    const int t = n_tok - keep + j;                             // the step's token that lands in place j
+    float v;
+    if (t >= 0) v = load_as_float(proj + (int64_t)(row0 + t) * proj_stride + x_col + ch) + x_bias[ch];
+    else v = old[j + n_tok];                                    // fewer new tokens than places: the old ones move up
+    tl[(int64_t)j * width] = v;
+  }
+}
+
+DRYFT_API int dryft_rglru_gates(const void* proj, int64_t proj_stride, int x_col, const float* x_bias,
+                                const float* conv_w, const float* conv_b, int taps, const void* gate_a,
+                                const float* gate_a_bias, const void* gate_i, const float* gate_i_bias,
+                                const float* lam, float decay_scale, const int* row_slot, const int* row_seq,
+                                const int* row_pos, const int* seq_start, const float* tail, float* coef, int n_rows,
+                                int width, int blocks, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (blocks <= 0 || width % blocks || taps < 1 || taps > RG_MAX_TAPS) return -1;
+  const int block_size = width / blocks;
+  const size_t lds = (size_t)RG_ROWS * block_size * sizeof(float);
+  if (lds > 64 * 1024) return -1;
+  dim3 grid((n_rows + RG_ROWS - 1) / RG_ROWS, blocks), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(rglru_gates_kernel<float>, grid, block, lds, stream, (const float*)proj, proj_stride, x_col,
+                       x_bias, conv_w, conv_b, taps, (const float*)gate_a, gate_a_bias, (const float*)gate_i,
+                       gate_i_bias, lam, decay_scale, row_slot, row_seq, row_pos, seq_start, tail, coef, n_rows, width,
+                       block_size);
+  else
+    hipLaunchKernelGGL(rglru_gates_kernel<bf16_t>, grid, block, lds, stream, (const bf16_t*)proj, proj_stride, x_col,
+                       x_bias, conv_w, conv_b, taps, (const bf16_t*)gate_a, gate_a_bias, (const bf16_t*)gate_i,
+                       gate_i_bias, lam, decay_scale, row_slot, row_seq, row_pos, seq_start, tail, coef, n_rows, width,
+                       block_size);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+DRYFT_API int dryft_rglru_scan(const float* coef, const void* proj, int64_t proj_stride, int x_col, int y_col,
+                               const float* x_bias, const float* y_bias, int taps, const int* seq_slot,
+                               const int* cu_rows, const int* q_len, const int* row_slot, int n_seqs, float* state,
+                               float* tail, void* out, int n_rows, int width, int write_state, int is_f32,
+                               hipStream_t stream) {
+  if (n_seqs <= 0 || n_rows <= 0) return 0;
+  if (taps < 1 || taps > RG_MAX_TAPS) return -1;
+  dim3 grid(n_seqs, (width + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, block, 0, stream, coef, (const float*)proj, proj_stride, x_col,
+                       y_col, x_bias, y_bias, taps, seq_slot, cu_rows, q_len, row_slot, state, tail, (float*)out,
+                       n_rows, width, write_state);
+  else
+    hipLaunchKernelGGL(rglru_scan_kernel<bf16_t>, grid, block, 0, stream, coef, (const bf16_t*)proj, proj_stride,
+                       x_col, y_col, x_bias, y_bias, taps, seq_slot, cu_rows, q_len, row_slot, state, tail,
+                       (bf16_t*)out, n_rows, width, write_state);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -491,3 +491,85 @@ DRYFT_API int dryft_qk_norm_rope_kv(const void* qkv, int64_t qkv_stride, const v
                        max_pages, n_rows, n_kv, head_dim);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// Rotary positions over neighbouring pairs, with float tables, and the append to the paged cache, for
+// heads whose keys and values may differ in width. Of the first `rot` features of every q and k head,
+// feature 2i and feature 2i + 1 turn together:
+//
+//   o[2i] = x[2i] c - x[2i+1] s,   o[2i+1] = x[2i+1] c + x[2i] s,   c = cos_t[pos, i], s = sin_t[pos, i]
+//
+// in float, rounded once; features from `rot` on pass. The tables are float32 [positions, rot/2] whatever
+// the activation dtype (the angle of a far position does not survive 8 bits of mantissa), and carry any
+// factor the encoding puts on both cos and sin. The row's q, k and v start at columns q_col, k_col and
+// v_col of `proj` (a fused projection that may hold more). One wave per head; lane l takes pairs l, l + 64, ...
+template <typename T>
+__global__ __launch_bounds__(256) void rope_pairs_kv_kernel(const T* __restrict__ proj, int64_t proj_stride, int q_col,
+                                                            int k_col, int v_col, const float* __restrict__ cos_t,
+                                                            const float* __restrict__ sin_t, int rot,
+                                                            const int* __restrict__ row_slot,
+                                                            const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                            T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                                            const int* __restrict__ page_table, int max_pages,
+                                                            int write_kv, int n_heads, int n_kv, int head_dim,
+                                                            int v_dim) {
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int64_t row = blockIdx.x;
+  const int job = blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
+  if (job >= n_heads + 2 * n_kv) return;
+  const int slot = row_slot[row], pos = row_pos[row];
+  const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
+  if (is_q) {
+    T* dst = q_out + (row * n_heads + job) * head_dim;
+    if (slot < 0) {
+      for (int i = lane; i < head_dim; i += WAVE) store_from_float(dst + i, 0.f);
+      return;
+    }
+  } else if (slot < 0 || !write_kv) {
+    return;
+  }
+  int page = 0, in_page = 0;
+  if (!is_q) {
+    page = page_of(page_table, max_pages, slot, pos);
+    in_page = pos % PAGE_TOKENS;
+    if (page < 0) return;  // no page: the host reserves one before the step; never write through a bad index
+  }
+  if (!is_q && !is_k) {
+    const int kvh = job - n_heads - n_kv;
+    const T* src = proj + row * proj_stride + v_col + (int64_t)kvh * v_dim;
+    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * v_dim * PAGE_TOKENS + value_column(in_page);
+    for (int i = lane; i < v_dim; i += WAVE) dst[(int64_t)i * PAGE_TOKENS] = src[i];
+    return;
+  }
+  const T* src = proj + row * proj_stride + (is_q ? q_col + (int64_t)job * head_dim
+                                                 : k_col + (int64_t)(job - n_heads) * head_dim);
+  T* dst = is_q ? q_out + (row * n_heads + job) * head_dim
+                : k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + in_page) * head_dim;
+  const int half = rot / 2;
+  for (int i = lane; i < half; i += WAVE) {
+    const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
+    const float a = load_as_float(src + 2 * i), b = load_as_float(src + 2 * i + 1);
+    store_from_float(dst + 2 * i, a * c - b * s);
+    store_from_float(dst + 2 * i + 1, b * c + a * s);
+  }
+  for (int i = rot + lane; i < head_dim; i += WAVE) dst[i] = src[i];
+}
+
+DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_col, int k_col, int v_col,
+                                  const float* cos_t, const float* sin_t, int rot, const int* row_slot,
+                                  const int* row_pos, void* q_out, void* k_pages, void* v_pages,
+                                  const int* page_table, int max_pages, int write_kv, int n_rows, int n_heads,
+                                  int n_kv, int head_dim, int v_dim, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (rot < 0 || rot % 2 || rot > head_dim || n_kv <= 0 || q_out == nullptr) return -1;
+  dim3 grid(n_rows, (n_heads + 2 * n_kv + 3) / 4), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(rope_pairs_kv_kernel<float>, grid, block, 0, stream, (const float*)proj, proj_stride, q_col,
+                       k_col, v_col, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages,
+                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim);
+  else
+    hipLaunchKernelGGL(rope_pairs_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)proj, proj_stride, q_col,
+                       k_col, v_col, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out, (bf16_t*)k_pages,
+                       (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -147,8 +147,8 @@ class Engine:
                 f"cache {self.cache.bytes() / 2**30:.2f} GiB for {self.max_tokens} tokens")
 
     # ------------------------------------------------------------------ the step function
-    def step(self, seqs: list[SeqStep]) -> torch.Tensor:
-        return self.stepper.step(seqs)
+    def step(self, seqs: list[SeqStep], tap=None) -> torch.Tensor:
+        return self.stepper.step(seqs, tap=tap)
 
     def tune(self, row_counts: Sequence[int]) -> None:
         """Lets the vendor library choose its kernels for steps of these many rows (a prompt of 2,048 tokens is a

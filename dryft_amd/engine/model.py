@@ -12,7 +12,7 @@ import torch
 
 from ..config.plan import ModelPlan
 from ..parts import block_class, build_part
-from ..parts.base import Partials, StepContext
+from ..parts.base import Deferred, Partials, StepContext
 from ..weights.spec import TensorSpec
 from ..csrc import ops
 
@@ -27,6 +27,7 @@ class DecoderModel:
         self.final_norm = build_part(plan.final_norm)
         self.head = build_part(plan.head)
         self.positions = {name: build_part(spec) for name, spec in plan.positions.items()}
+        self.stream_parts = {name: build_part(spec) for name, spec in plan.stream_parts.items()}
         self.blocks = []
         self._bindings: list[tuple[object, dict[str, str]]] = []   # (part, logical -> checkpoint name)
         self._bindings.append((self.embedding, plan.embedding.tensors))
@@ -43,6 +44,10 @@ class DecoderModel:
         self._bindings.append((self.head, plan.head.tensors))
         for name, part in self.positions.items():
             self._bindings.append((part, plan.positions[name].tensors))
+        for name, part in self.stream_parts.items():
+            self._bindings.append((part, plan.stream_parts[name].tensors))
+        for part, _ in self._bindings:
+            part.compute_dtype = dtype
 
     # ---- what the model wants from a checkpoint
     def tensor_specs(self) -> list[TensorSpec]:
@@ -135,15 +140,22 @@ class DecoderModel:
             part.prepare(n_positions, self.dtype, self.device)
 
     # ---- compute
-    def forward(self, tokens: torch.Tensor, ctx: StepContext, cache, rows: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, ctx: StepContext, cache, rows: torch.Tensor | None = None,
+                tap=None) -> torch.Tensor:
         """Hidden states after the final norm, ``[rows, hidden]``: of every row of the step, or of ``rows`` alone
         (int32 indices into the step's rows, on the device), which are picked before the final norm so that it runs
-        over nothing else."""
+        over nothing else. ``tap(i, stream)``, when given, is called after run ``i`` of the schedule with the residual
+        stream as that run leaves it (float32, everything pending added): a way to look, not part of the step."""
         ctx.positions = self.positions
         x = self.embedding.forward(tokens)
+        ctx.embedded = x
         pending = None
-        for run in self.plan.schedule:
+        for i, run in enumerate(self.plan.schedule):
+            if run.enter is not None:
+                pending = self.stream_parts[run.enter[0]].enter(pending, run.enter[1], ctx)
             x, pending = self.blocks[run.layer].forward(x, pending, ctx, cache.line(run.cache_line), run.writes_cache)
+            if tap is not None:
+                tap(i, _settled(x, pending))
         if rows is not None:
             if rows.numel() == 0:                              # nothing is wanted: the layers have run, that is all
                 return x[:0]
@@ -158,11 +170,24 @@ class DecoderModel:
         return self.head.forward(hidden if rows is None else _pick_rows(hidden, rows))
 
 
+def _settled(x: torch.Tensor, pending) -> torch.Tensor:
+    """The residual stream with what is pending added, float32."""
+    if isinstance(pending, Deferred) or x.dtype == torch.float32 and pending is not None:
+        from ..parts.stream import settle
+        return settle(x, pending)
+    if pending is None:
+        return x.float()
+    delta = pending.summed(torch.float32) if isinstance(pending, Partials) else pending.float()
+    return (x.float() + delta).to(x.dtype).float()
+
+
 def _pick_rows(x, rows: torch.Tensor):
     """Rows ``rows`` of a tensor ``[n, width]`` or of partial sums ``[count, n, width]`` (a row gather is what the
     embedding kernel does)."""
     if x is None:
         return None
+    if isinstance(x, Deferred):
+        return x.picked(lambda t: _pick_rows(t, rows))
     if isinstance(x, Partials):
         parts = x.data[:x.count]
         picked = torch.empty((x.count, rows.numel(), parts.shape[2]), dtype=parts.dtype, device=parts.device)

@@ -115,8 +115,9 @@ class Stepper:
             self._buffers = b
         return b
 
-    def step(self, seqs: list[SeqStep]) -> torch.Tensor:
-        """Runs the step and returns float32 logits ``[sum(len(want)), vocab]`` in order."""
+    def step(self, seqs: list[SeqStep], tap=None) -> torch.Tensor:
+        """Runs the step and returns float32 logits ``[sum(len(want)), vocab]`` in order. ``tap``: see
+        ``DecoderModel.forward``."""
         if not seqs:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)
         tokens: list[int] = []
@@ -139,7 +140,7 @@ class Stepper:
         ctx = stage_batch(self.cache, buf, slots, q_lens, tok, self.model.dtype)
         # the wanted rows are picked before the final norm; when every row is wanted in order, nothing is picked
         rows = None if wanted == list(range(ctx.n_rows)) else torch.tensor(wanted, dtype=torch.int32, device=self.device)
-        hidden = self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache, rows)
+        hidden = self.model.forward(buf.tokens[:ctx.n_rows], ctx, self.cache, rows, tap=tap)
         self.cache.end_step([s for s in slots if s >= 0], [q for s, q in zip(slots, q_lens) if s >= 0])
         if not wanted:
             return torch.empty((0, self.vocab), dtype=torch.float32, device=self.device)

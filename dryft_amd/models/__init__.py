@@ -42,6 +42,8 @@ def known_architectures() -> list[str]:
 
 def resolve_architecture(raw_config: dict[str, Any]) -> Architecture:
     names = raw_config.get("architectures")
+    if names is None and isinstance(raw_config.get("architecture"), str):
+        names = [raw_config["architecture"]]                        # a config.json that names one class, as a string
     if names is None and raw_config.get("model_type") in _MODEL_TYPES:
         names = [_MODEL_TYPES[raw_config["model_type"]]]          # a config.json that only says model_type
     if not isinstance(names, list) or not names or not isinstance(names[0], str):
@@ -72,3 +74,4 @@ def load_preset(name: str) -> dict:
 
 
 from . import qwen3 as _qwen3  # noqa: E402,F401  (registers Qwen3ForCausalLM)
+from . import piralix as _piralix  # noqa: E402,F401  (registers Piralix)

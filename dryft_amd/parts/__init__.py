@@ -8,7 +8,8 @@ by a plan.
 
 from __future__ import annotations
 
-from .base import (FeedForward, HostBatch, Mixer, Norm, Part, Partials, PositionEncoding, StepContext, matrix)
+from .base import (Deferred, FeedForward, HostBatch, Mixer, Norm, Part, Partials, PositionEncoding, StepContext,
+                   StreamPart, matrix)
 
 _PARTS: dict[str, type] = {}
 _BLOCKS: dict[str, type] = {}
@@ -44,7 +45,7 @@ def build_part(spec) -> Part:
     return part_class(spec.kind)(**spec.args)
 
 
-from . import attention, block, embedding, mlp, norm, rope  # noqa: E402,F401  (register the built-in parts)
+from . import attention, block, embedding, mlp, norm, recurrent, rope, stream  # noqa: E402,F401  (register the built-in parts)
 
-__all__ = ["FeedForward", "HostBatch", "Mixer", "Norm", "Part", "Partials", "PositionEncoding", "StepContext", "matrix",
+__all__ = ["Deferred", "StreamPart", "FeedForward", "HostBatch", "Mixer", "Norm", "Part", "Partials", "PositionEncoding", "StepContext", "matrix",
            "register_part", "register_block", "part_class", "block_class", "build_part"]

@@ -7,6 +7,13 @@ causal scores ``(q . k) / sqrt(head_dim)`` against every cached key of the seque
 own position (or the last ``window`` of them), query head ``h`` reading kv head ``h // group``
 (model.py:172-177, 254-257); output projection (model.py:179). No biases.
 
+Options other designs use, all off by default: values of another width than the keys (``value_dim``); a
+capped score, ``s <- softcap * tanh(s / softcap)``; a sink per query head (tensor ``sink``), whose ``exp`` joins
+the softmax's denominator and nothing else; an output gate, the heads' outputs times ``sigmoid(W_g h)`` before
+the output projection (tensor ``g_proj``, fused into the q/k/v product); attention weights kept in float
+(``float_weights``); and, when the position encoding it names rotates neighbouring pairs
+(``PairRotaryPositions``), that rotation with float tables. Any of these takes the step down ``_forward_general``.
+
 The part knows nothing of the model around it: sizes and constants are constructor arguments, the
 position encoding is looked up by name in the step context, and its storage is the cache line it
 is handed.
@@ -26,6 +33,7 @@ from ..weights.spec import VECTOR
 from . import register_part
 from .base import Mixer, Partials, StepContext, matrix
 from .linear import linear
+from .rope import PairRotaryPositions
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
@@ -36,7 +44,9 @@ _PROMPT_PARTIAL_ROWS = 256      # and so do prompt steps of at most so many rows
 class GQAAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None = None, positions: str | None = None, rotary_dim: int | None = None,
-                 window: int | None = None, scale: float | None = None):
+                 window: int | None = None, scale: float | None = None, value_dim: int | None = None,
+                 softcap: float | None = None, sink: bool = False, output_gate: bool = False,
+                 float_weights: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
         if not 0 < head_dim <= MAX_HEAD_DIM:
@@ -49,19 +59,37 @@ class GQAAttention(Mixer):
             raise ValueError(f"the rotated width must be even and at most head_dim ({head_dim}), got {self.rotary_dim}")
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # model.py:65
+        self.value_dim = int(value_dim) if value_dim else self.head_dim
+        if not 0 < self.value_dim <= MAX_HEAD_DIM:
+            raise ValueError(f"value_dim must lie in 1..{MAX_HEAD_DIM}, got {value_dim}")
+        self.softcap = float(softcap) if softcap else 0.0
+        self.has_sink, self.output_gate, self.float_weights = bool(sink), bool(output_gate), bool(float_weights)
         self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
-        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+        self.v_dim, self.o_dim = self.n_kv * self.value_dim, self.n_heads * self.value_dim
+        self.extended = bool(self.value_dim != self.head_dim or self.softcap or self.has_sink or self.output_gate or
+                             self.float_weights)
+        if self.extended and self.qk_norm_eps is not None:
+            raise ValueError("per-head q/k norms are not combined with a capped score, a sink, an output gate or "
+                             "values of another width")
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.sink = None
 
     def tensor_specs(self):
         specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
-                 "v_proj": matrix((self.kv_dim, self.hidden)), "o_proj": matrix((self.hidden, self.q_dim))}
+                 "v_proj": matrix((self.v_dim, self.hidden)), "o_proj": matrix((self.hidden, self.o_dim))}
+        if self.has_sink:
+            specs["sink"] = ((self.n_heads,), VECTOR, "normal")
+        if self.output_gate:
+            specs["g_proj"] = matrix((self.o_dim, self.hidden))
         if self.qk_norm_eps is not None:
             specs["q_norm"] = ((self.head_dim,), VECTOR, "ones")
             specs["k_norm"] = ((self.head_dim,), VECTOR, "ones")
         return specs
 
     def load(self, tensors):
-        self.w_qkv = torch.cat([tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]], dim=0).contiguous()
+        fused = [tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]] + ([tensors["g_proj"]] if self.output_gate else [])
+        self.w_qkv = torch.cat(fused, dim=0).contiguous()
+        if self.has_sink:
+            self.sink = tensors["sink"].float().contiguous()
         self.w_o = tensors["o_proj"]
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm"], tensors["k_norm"]
@@ -69,12 +97,43 @@ class GQAAttention(Mixer):
                 self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
 
     def cache_need(self):
-        return KVNeed(self.n_kv, self.head_dim, self.window)
+        return KVNeed(self.n_kv, self.head_dim, self.window,
+                      self.value_dim if self.value_dim != self.head_dim else None)
 
     def kernel_modules(self, dtype):
         return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ())
 
+    def _forward_general(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
+        """Every option, in float arithmetic on the kernel that takes one (row, head) a workgroup."""
+        rows, H, G, D, Dv = h.shape[0], self.n_heads, self.n_kv, self.head_dim, self.value_dim
+        cos = sin = None
+        rot = 0
+        if self.positions:
+            table = ctx.positions[self.positions]
+            if not isinstance(table, PairRotaryPositions):
+                raise NotImplementedError("the options of this attention go with a rotation over neighbouring pairs")
+            if ctx.max_kv_len > table.n_positions:
+                raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
+            cos, sin, rot = table.cos, table.sin, table.dims
+            if rot > D:
+                raise ValueError(f"the position encoding rotates {rot} features, a head has {D}")
+        proj = linear(h, self.w_qkv)                                    # q | k | v | gate
+        q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
+        ops.rope_pairs_kv(proj, 0, self.q_dim, self.q_dim + self.kv_dim, cos, sin, rot, ctx.row_slot, ctx.row_pos, q,
+                          line.k, line.v, line.page_table, writes_cache, H, G, D, Dv)
+        out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
+        ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
+                      self.window or 0, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights)
+        out = out.view(rows, self.o_dim)
+        if self.output_gate:
+            gated = torch.empty_like(out)
+            g_col = self.q_dim + self.kv_dim + self.v_dim
+            out = ops.sigmoid_gate(out, proj[:, g_col:g_col + self.o_dim], gated)
+        return linear(out, self.w_o, allow_partials=True)
+
     def forward(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
+        if self.extended or (self.positions and isinstance(ctx.positions[self.positions], PairRotaryPositions)):
+            return self._forward_general(h, ctx, line, writes_cache)
         rows = h.shape[0]
         # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
         matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0
@@ -171,7 +230,7 @@ class GQAAttention(Mixer):
                 seen += (2 * first + full - 1) * full // 2 + (q - full) * self.window
             else:
                 seen += (first + last) * q // 2
-        return super().flops(rows, spans) + 4.0 * self.q_dim * seen
+        return super().flops(rows, spans) + 2.0 * (self.q_dim + self.o_dim) * seen
 
     def decode_splits(self, n_seqs: int, max_kv_len: int) -> int:
         """How many ways each sequence's keys are split: as many as run at the same time, and no more.

@@ -57,6 +57,7 @@ class StepContext:
     max_kv_len: int                     # host bound on any sequence's cached length after the step
     host: HostBatch | None = None
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
+    embedded: torch.Tensor | None = None    # the embedding's output of this step's rows, for parts that come back to it
     _tiles: dict[int, tuple[torch.Tensor, int]] = field(default_factory=dict, repr=False)
     _kept: dict[Any, torch.Tensor] = field(default_factory=dict, repr=False)
 
@@ -114,8 +115,27 @@ class Partials:
         return ops.sum_partials(self.data, out, self.count)
 
 
+@dataclass
+class Deferred:
+    """What has still to be added to a float32 residual stream before the next norm reads it, so that one kernel
+    can do all of it: a branch's output ``delta`` (a tensor or ``Partials``) that is normed with ``norm`` first (None:
+    added as it is), a tensor ``rows`` in the activation dtype that is added row by row (the embedding's output coming
+    back), and a ``vector`` added to every row."""
+
+    delta: Any = None
+    norm: Any = None
+    rows: torch.Tensor | None = None
+    vector: torch.Tensor | None = None
+
+    def picked(self, pick) -> "Deferred":
+        """The same for a choice of rows; ``pick`` gathers them from a tensor or from partial sums."""
+        return Deferred(pick(self.delta), self.norm, pick(self.rows), self.vector)
+
+
 class Part:
     """Base of all parts. ``tensor_specs`` maps logical names to (shape, role, init)."""
+
+    compute_dtype: torch.dtype | None = None    # the dtype the model computes in, set by the model that builds the part
 
     def tensor_specs(self) -> dict[str, tuple[tuple[int, ...], str, str]]:
         return {}
@@ -167,6 +187,16 @@ class Mixer(Part):
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, ctx: StepContext):
+        raise NotImplementedError
+
+
+class StreamPart(Part):
+    """Acts on the residual stream between two runs of the schedule (where a pass over a run of layers begins, say):
+    a run that names it hands over what is still to be added to the stream and gets back what is to be added now."""
+
+    def enter(self, pending, index: int, ctx: StepContext):
+        """``pending`` is what the run before left (None, a tensor, ``Partials`` or ``Deferred``); ``index`` is the
+        number the schedule gives this entry. Returns the new pending."""
         raise NotImplementedError
 
 

@@ -44,4 +44,32 @@ class SwiGLU(FeedForward):
         return linear(act, self.w_down, allow_partials=True)
 
 
+class ClampedGLU(FeedForward):
+    """``down( g * sigmoid(alpha * g) * (u + 1) )`` with ``g = min(gate(h), limit)`` and
+    ``u = clamp(up(h), -limit, limit)``, dense, no bias. Gate and up are one product, as above."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702):
+        self.hidden, self.inter = int(hidden_size), int(intermediate_size)
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.w_gate_up: torch.Tensor | None = None
+        self.w_down: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return {"gate_proj": matrix((self.inter, self.hidden)), "up_proj": matrix((self.inter, self.hidden)),
+                "down_proj": matrix((self.hidden, self.inter))}
+
+    def load(self, tensors):
+        self.w_gate_up = torch.cat([tensors["gate_proj"], tensors["up_proj"]], dim=0).contiguous()
+        self.w_down = tensors["down_proj"]
+
+    def kernel_modules(self, dtype):
+        return ("gemm", "activation")
+
+    def forward(self, h, ctx):
+        act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
+        ops.glu_clamped(linear(h, self.w_gate_up), act, self.limit, self.alpha)
+        return linear(act, self.w_down, allow_partials=True)
+
+
 register_part("swiglu", SwiGLU)
+register_part("clamped_glu", ClampedGLU)

@@ -11,6 +11,8 @@ would use, then uploaded.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from . import register_part
@@ -37,4 +39,51 @@ class RotaryPositions(PositionEncoding):
         self.n_positions = n_positions
 
 
+class PairRotaryPositions(PositionEncoding):
+    """Rotary tables for a rotation over neighbouring pairs ``(2i, 2i + 1)`` of the first ``dims`` features, kept in
+    float32 whatever the activation dtype: ``cos``/``sin`` are ``[positions, dims / 2]`` of the angles
+    ``p * f_i``, ``f_i = base^(-2i / dims)``.
+
+    With ``scaling`` (YaRN: ``factor``, ``original`` context length, ``fast`` and ``slow`` turn counts) the slow
+    pairs are stretched and the fast ones left alone: with ``d(t) = dims * ln(original / (2 pi t)) / (2 ln base)``,
+    ``lo = max(floor(d(fast)), 0)``, ``hi = min(ceil(d(slow)), dims - 1)`` and
+    ``ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)`` the frequency becomes
+    ``f_i / factor * ramp_i + f_i * (1 - ramp_i)``, and cos and sin are both multiplied by ``0.1 ln(factor) + 1``
+    (the tables carry that factor). Angles are formed in float64 on the host and rounded once."""
+
+    def __init__(self, dims: int, base: float, scaling: dict | None = None):
+        if dims % 2 or dims < 0:
+            raise ValueError(f"the rotated width must be even, got {dims}")
+        self.dims, self.base = int(dims), float(base)
+        self.scaling = dict(scaling) if scaling else None
+        self.cos: torch.Tensor | None = None
+        self.sin: torch.Tensor | None = None
+        self.n_positions = 0
+
+    def frequencies(self) -> tuple[torch.Tensor, float]:
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        f = self.base ** (-2.0 * i / max(self.dims, 1))
+        if not self.scaling:
+            return f, 1.0
+        factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+
+        def pair_of(turns: float) -> float:
+            return self.dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+
+        lo = max(math.floor(pair_of(float(self.scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(self.scaling["slow"]))), self.dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        return f / factor * ramp + f * (1 - ramp), 0.1 * math.log(factor) + 1.0
+
+    def prepare(self, n_positions: int, dtype: torch.dtype, device) -> None:
+        if self.cos is not None and n_positions <= self.n_positions:
+            return
+        f, both = self.frequencies()
+        angle = torch.arange(n_positions, dtype=torch.float64)[:, None] * f[None, :]
+        self.cos = (angle.cos() * both).to(torch.float32).to(device).contiguous()
+        self.sin = (angle.sin() * both).to(torch.float32).to(device).contiguous()
+        self.n_positions = n_positions
+
+
 register_part("rotary", RotaryPositions)
+register_part("pair_rotary", PairRotaryPositions)

@@ -1,0 +1,151 @@
+"""A float32 residual stream with a norm on both sides of every branch.
+
+``x <- x + norm_b(branch(norm_a(x)))``: the branch's output is normed before it is added, and the stream is
+normed again for the next branch. The stream stays float32 whatever the activation dtype, so that the sum
+over many layers (and over several passes through the same layers) is not rounded to 8 bits each time.
+Every residual sum is folded into the norm that follows it: a block hands its last branch's output on
+unadded (``Deferred``), and the next block's first kernel norms it, adds it, adds whatever else has come
+due meanwhile, and norms the stream for its own first branch, in one launch.
+
+``StreamRMSNorm``    the norm itself: ``x / sqrt(mean(x^2) + eps) * w`` in float, rounded once.
+``SandwichBlock``    mixer and feed-forward, each between two norms; ``SandwichMixerBlock`` has the mixer alone.
+``PassEntry``        what a pass over a run of layers begins with: one learned vector per pass is added to the
+                     stream, and from the second pass on the embedding's output once more.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..csrc import ops
+from ..weights.spec import VECTOR
+from . import register_block, register_part
+from .base import Deferred, FeedForward, Mixer, Norm, Partials, StepContext, StreamPart
+
+
+class StreamRMSNorm(Norm):
+    def __init__(self, size: int, eps: float):
+        self.size, self.eps = int(size), float(eps)
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return {"weight": ((self.size,), VECTOR, "ones")}
+
+    def load(self, tensors):
+        self.weight = tensors["weight"].float()
+
+    def kernel_modules(self, dtype):
+        return ("norm",)
+
+    def forward(self, x: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+        y = torch.empty(x.shape, dtype=dtype or self.compute_dtype or x.dtype, device=x.device)
+        ops.stream_norm(x, None, None, None, None, self.weight, self.eps, None, y, y.dtype)
+        return y
+
+    def add_forward(self, res: torch.Tensor, delta, dtype: torch.dtype | None = None, in_place: bool = True):
+        """``(stream, norm(stream))`` after everything in ``delta`` (a ``Deferred``, a tensor, ``Partials`` or None)
+        has been added to ``res``. The stream comes back as float32: ``res`` itself, updated, when it is float32 and
+        ``in_place`` allows; the normed rows in ``dtype`` (default: the dtype the model computes in)."""
+        pending = as_deferred(delta)
+        act = dtype or self.compute_dtype or _activation_dtype(res, pending)
+        own = in_place and res.dtype == torch.float32 and res.is_contiguous()
+        out = res if own else torch.empty(res.shape, dtype=torch.float32, device=res.device)
+        y = torch.empty(res.shape, dtype=act, device=res.device)
+        _launch(res, pending, self.weight, self.eps, out, y, act)
+        return out, y
+
+
+def as_deferred(pending) -> Deferred:
+    if pending is None:
+        return Deferred()
+    if isinstance(pending, Deferred):
+        return pending
+    return Deferred(delta=pending)
+
+
+def _activation_dtype(x: torch.Tensor, pending: Deferred) -> torch.dtype:
+    for t in (pending.delta, pending.rows):
+        if isinstance(t, torch.Tensor):
+            return t.dtype
+    return x.dtype
+
+
+def _launch(x, pending: Deferred, weight, eps, x_out, y, act) -> None:
+    delta = pending.delta
+    if isinstance(delta, Partials):
+        delta = (delta.data, delta.count)
+    post = pending.norm.weight if pending.norm is not None else None
+    if pending.norm is not None and pending.norm.eps != eps:
+        raise ValueError("the norms around one residual sum differ in eps; one launch takes one")
+    ops.stream_norm(x, delta, post, pending.rows, pending.vector, weight, eps, x_out, y, act)
+
+
+def settle(x: torch.Tensor, pending, eps: float = 0.0) -> torch.Tensor:
+    """The stream with everything pending added, as a new float32 tensor (for looking at it; the compute path never
+    needs the stream without the norm that follows)."""
+    pending = as_deferred(pending)
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    act = _activation_dtype(x, pending)
+    _launch(x, pending, None, pending.norm.eps if pending.norm is not None else eps, out, None, act)
+    return out
+
+
+class SandwichBlock:
+    roles = ("mixer_norm", "mixer", "mixer_post_norm", "ffn_norm", "ffn", "ffn_post_norm")
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_post_norm: Norm, ffn_norm: Norm | None = None,
+                 ffn: FeedForward | None = None, ffn_post_norm: Norm | None = None):
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ffn_norm, self.ffn, self.ffn_post_norm = ffn_norm, ffn, ffn_post_norm
+
+    def parts(self):
+        return {role: getattr(self, role) for role in self.roles}
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache: bool):
+        # the embedding's output starts the stream and is read again later: it is never updated in place
+        x, h = self.mixer_norm.add_forward(x, pending, ctx.dtype, in_place=x is not ctx.embedded)
+        pending = Deferred(delta=self.mixer.forward(h, ctx, line, writes_cache), norm=self.mixer_post_norm)
+        if self.ffn is None:
+            return x, pending
+        x, h = self.ffn_norm.add_forward(x, pending, ctx.dtype)
+        return x, Deferred(delta=self.ffn.forward(h, ctx), norm=self.ffn_post_norm)
+
+
+class SandwichMixerBlock(SandwichBlock):
+    roles = ("mixer_norm", "mixer", "mixer_post_norm")
+
+
+class PassEntry(StreamPart):
+    """``steps [passes, width]``: pass ``t`` begins by adding ``steps[t]`` to every row of the stream, and every pass
+    but the first (when ``readd_embedding``) by adding the embedding's output of the row once more."""
+
+    def __init__(self, passes: int, size: int, readd_embedding: bool = True):
+        self.passes, self.size, self.readd = int(passes), int(size), bool(readd_embedding)
+        self.steps: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return {"steps": ((self.passes, self.size), VECTOR, "normal")}
+
+    def load(self, tensors):
+        self.steps = tensors["steps"].float().contiguous()
+
+    def kernel_modules(self, dtype):
+        return ("norm",)
+
+    def reads_whole(self) -> bool:
+        return False
+
+    def enter(self, pending, index: int, ctx: StepContext) -> Deferred:
+        if not 0 <= index < self.passes:
+            raise ValueError(f"pass {index} of {self.passes}")
+        pending = as_deferred(pending)
+        if pending.rows is not None or pending.vector is not None:
+            raise ValueError("two entries before one run")
+        rows = ctx.embedded if self.readd and index > 0 else None
+        return Deferred(pending.delta, pending.norm, rows, self.steps[index])
+
+
+register_part("stream_rmsnorm", StreamRMSNorm)
+register_part("pass_entry", PassEntry)
+register_block("sandwich", SandwichBlock)
+register_block("sandwich_mixer", SandwichMixerBlock)
