@@ -23,13 +23,16 @@ import sys
 import numpy as np
 
 
+MAX_LIVE_REQUESTS = 128      # slots the replay program opens (fewer when the token budget allows fewer requests)
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
     ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time, each request rounded up to a whole cache page")
+                    help="most tokens live requests hold at any time")
     return ap
 
 
@@ -65,14 +68,16 @@ def main(argv=None) -> int:
     from .engine import Engine
 
     os.makedirs(args.out, exist_ok=True)
-    # the budget in whole pages; one request may take all of it, up to what the model allows
+    # The budget counts tokens, the cache whole pages: a request's last page may be partly empty, so every slot gets
+    # one page beyond the budget's own. One request may take all of it, up to what the model allows.
     pages = max(1, pages_for(args.max_tokens))
+    slots = max(1, min(args.max_tokens, MAX_LIVE_REQUESTS))
     raw = read_config_json(args.model)
     arch = resolve_architecture(raw)
     limit = arch.plan(arch.config_class.from_dict(raw)).max_positions
     max_len = min(pages * PAGE_TOKENS, limit) if limit else pages * PAGE_TOKENS
-    engine = Engine(args.model, dtype=args.dtype, max_batch=min(pages, 4096), max_len=max_len,
-                    max_tokens=pages * PAGE_TOKENS, use_graph=False)
+    engine = Engine(args.model, dtype=args.dtype, max_batch=slots, max_len=max_len,
+                    max_tokens=(pages + slots) * PAGE_TOKENS, use_graph=False)
     replayer = Replayer(engine)
     for line in sys.stdin:
         line = line.strip()
