@@ -36,6 +36,30 @@ __device__ __forceinline__ __bf16 to_bf16(float f) { return (__bf16)f; }
 // 2^x by the hardware instruction alone: arguments here are <= 0 or -inf, results below the normal range may flush to 0
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// tanh(x) = 1 - 2 / (1 + e^(2x)), from the hardware's exp2 and reciprocal: e^(2x) = inf gives 1, 0 gives -1
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * 2.88539008177792681472f));
+}
+
+// Options of the score that some designs use. A cap: s <- cap * tanh(s * scale / cap) (`pre` = scale / cap; 0: none).
+// A sink: one float per query head whose exp() joins the softmax's denominator and nothing else (null: none).
+struct ScoreCap {
+  float cap = 0.f, pre = 0.f;
+};
+struct ScoreOptions {
+  float softcap;
+  const float* sink;
+};
+__device__ __forceinline__ ScoreCap score_cap(const ScoreOptions& o, float scale) {
+  ScoreCap c;
+  if (o.softcap > 0.f) { c.cap = o.softcap; c.pre = scale / o.softcap; }
+  return c;
+}
+// 2^(sink in units of log2 e - m): what the sink adds to a row's sum whose reference maximum is m
+__device__ __forceinline__ float sink_term(const float* sink, int head, float m) {
+  return __builtin_amdgcn_exp2f(fminf(sink[head] * 1.44269504088896340736f - m, 126.f));
+}
+
 // State of one wave's 16 rows while it walks over pages of keys.
 template <int KB>  // KB = ceil(head_dim / 32)
 struct RowBlock {
@@ -130,8 +154,14 @@ __device__ __forceinline__ void page_scores(f32x4 (&s)[4], const PageK<KB>& f, c
 #define MAX_SLACK 8.f
 template <int KB, bool MASKED>
 __device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], bf16x8 (&p)[2], float scale_log2,
-                                              int key0, int lo_row, int hi_row, bool& moved) {
+                                              int key0, int lo_row, int hi_row, bool& moved, ScoreCap cap = {}) {
   const int g = (threadIdx.x % WAVE) / 16;
+  if (cap.cap > 0.f) {                                        // s <- cap * tanh(s * scale / cap); scale_log2 is log2(e) then
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[t][i] = cap.cap * fast_tanh(s[t][i] * cap.pre);
+  }
   float lane_max = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
@@ -191,21 +221,22 @@ __device__ __forceinline__ void page_values(RowBlock<KB>& st, const bf16x8 (&p)[
 
 template <int KB, bool MASKED>
 __device__ __forceinline__ void page_update_impl(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, float scale_log2,
-                                                 int key0, int lo_row, int hi_row) {
+                                                 int key0, int lo_row, int hi_row, ScoreCap cap) {
   bf16x8 p[2];
   bool moved;
-  const float alpha = page_softmax<KB, MASKED>(st, s, p, scale_log2, key0, lo_row, hi_row, moved);
+  const float alpha = page_softmax<KB, MASKED>(st, s, p, scale_log2, key0, lo_row, hi_row, moved, cap);
   page_values<KB>(st, p, alpha, moved, f);
 }
 
 // `masked` must be the same for all lanes of the wave.
 template <int KB>
 __device__ __forceinline__ void page_update(RowBlock<KB>& st, f32x4 (&s)[4], const PageV<KB>& f, int head_dim,
-                                            float scale_log2, int key0, int lo_row, int hi_row, bool masked = true) {
+                                            float scale_log2, int key0, int lo_row, int hi_row, bool masked = true,
+                                            ScoreCap cap = {}) {
   if (masked)
-    page_update_impl<KB, true>(st, s, f, scale_log2, key0, lo_row, hi_row);
+    page_update_impl<KB, true>(st, s, f, scale_log2, key0, lo_row, hi_row, cap);
   else
-    page_update_impl<KB, false>(st, s, f, scale_log2, key0, lo_row, hi_row);
+    page_update_impl<KB, false>(st, s, f, scale_log2, key0, lo_row, hi_row, cap);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -332,9 +363,10 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window, ScoreOptions opt) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int U = GP * RP, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP;
+  const ScoreCap cap = score_cap(opt, scale);
   // Two heads per wave: a workgroup takes one tile from each end of the list (grid: pairs of tiles x heads / 2).
   // Otherwise: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x tiles),
   // so that the short tiles fill the compute units that the long ones leave.
@@ -385,7 +417,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
   const int hi_wave = pos_wave + wave_rows - 1;               // below lo_wave for a wave without rows
   const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
   const int hi_tile = pos_tile + min(TILE_ROWS, q_len - tile_first) - 1;
-  const float scale_log2 = scale * 1.44269504088896340736f;
+  const float scale_log2 = (cap.cap > 0.f ? 1.f : scale) * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
   const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
@@ -440,8 +472,8 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
         // row, starts before a window's edge, or the tile has fewer than 16 rows
         const bool masked = key0 + PAGE_TOKENS - 1 > pos0[rt] || rows[rt] < 16 ||
                             (window > 0 && key0 < pos0[rt] + 15 - window + 1);
-        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u])
-                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u]);
+        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], cap)
+                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], cap);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -469,6 +501,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (!row_valid[u / GP]) continue;
+    if (opt.sink != nullptr) row_l[u] += sink_term(opt.sink, head0 + u % GP, st[u].m);
     const float inv = 1.f / row_l[u];
     bf16_t* o = out + (row[u / GP] * n_heads + head0 + u % GP) * head_dim;
 #pragma unroll
@@ -862,7 +895,8 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits,
-    FusedQKV fused, bf16_t* k_pages_w, bf16_t* v_pages_w, bf16_t* __restrict__ out) {
+    FusedQKV fused, bf16_t* k_pages_w, bf16_t* v_pages_w, bf16_t* __restrict__ out, ScoreOptions opt) {
+  const ScoreCap cap = score_cap(opt, scale);
   __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
   __shared__ float merge_ml[SPLIT_WAVES][16][2];
   __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][32 * KB];
@@ -888,7 +922,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     pg_first = pg_lo + split * per;
     pg = pg_first + wave;
   }
-  const float scale_log2 = scale * 1.44269504088896340736f;
+  const float scale_log2 = (cap.cap > 0.f ? 1.f : scale) * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   PageK<KB> kf;
   PageV<KB> vf;
@@ -997,7 +1031,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
       page_scores<KB>(s, kf, st);
       if (page_next >= 0)
         load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
-      page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo, pos);
+      page_update<KB>(st, s, vf, head_dim, scale_log2, pg * PAGE_TOKENS, lo, pos, true, cap);
     } else if (page_next >= 0) {
       load_page_k<KB, FULL>(kf, k_pages + ((int64_t)page_next * n_kv + kvh) * page_elems, head_dim);
     }
@@ -1032,6 +1066,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
       o += wgt * merge_o[w][r][d];
     }
     if (n_splits == 1) {                                   // nothing to combine: this is the result
+      if (opt.sink != nullptr && m != -INFINITY) l += sink_term(opt.sink, kvh * group + hb * 16 + r, m);
       out[(row * n_heads + kvh * group + hb * 16 + r) * head_dim + d] = float_to_bf16(l > 0.f ? o / l : 0.f);
       continue;
     }
@@ -1052,7 +1087,8 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const flo
                                                            const float* __restrict__ part_ml,
                                                            const int* __restrict__ seq_slot,
                                                            const int* __restrict__ cu_rows, bf16_t* __restrict__ out,
-                                                           int n_heads, int head_dim, int n_splits) {
+                                                           int n_heads, int head_dim, int n_splits,
+                                                           const float* __restrict__ sink) {
   __shared__ float wgt[COMBINE_MAX_SPLITS];
   __shared__ float inv_l;
   const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
@@ -1076,7 +1112,8 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_combine_kernel(const flo
     const float ls = (live && tid < n_splits) ? ml[2 * tid + 1] : 0.f;
     const float m = wave_max(ms);
     const float w = (ms == -INFINITY) ? 0.f : exp2f(ms - m);
-    const float l = wave_sum(w * ls);
+    float l = wave_sum(w * ls);
+    if (sink != nullptr && m != -INFINITY) l += sink_term(sink, head, m);
     if (tid < n_splits) wgt[tid] = w;
     if (tid == 0) inv_l = l > 0.f ? 1.f / l : 0.f;
   }
@@ -1115,7 +1152,7 @@ template <int GP, int RP>
 static int launch_causal(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
                          const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
                          int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window,
-                         hipStream_t stream) {
+                         ScoreOptions opt, hipStream_t stream) {
   dim3 grid((max_tiles + 1) / 2, n_heads / GP), block(256);
   // max_tiles bounds the 64-row tiles of the sequences that take part. Tiles of 128 rows: a sequence with t
   // 64-row tiles has (t + 1) / 2 of them, so all together at most (max_tiles + n_seqs) / 2.
@@ -1131,7 +1168,7 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
       return -1;                                                                                                   \
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,                 \
                        (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs, \
-                       (bf16_t*)out, n_heads, n_kv, head_dim, scale, window);                                      \
+                       (bf16_t*)out, n_heads, n_kv, head_dim, scale, window, opt);                                 \
   }
   if (head_dim % 32 == 0) {
     DISPATCH_KB(head_dim / 32, LAUNCH_CAUSAL(true));
@@ -1163,14 +1200,16 @@ static int launch_causal_direct(const void* q, const void* k_pages, const void* 
 static int causal_entry(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
                         const int* seq_slot, const int* cu_rows, const int* tile_cu, const int* seq_start, int n_seqs,
                         int max_tiles, void* out, int n_heads, int n_kv, int head_dim, float scale, int window, int mode,
-                        ProjectedQ projected, hipStream_t stream) {
+                        ProjectedQ projected, hipStream_t stream, ScoreOptions opt = {0.f, nullptr}) {
   if (n_seqs <= 0 || max_tiles <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim)) return -1;
   const int group = n_heads / n_kv;
   const bool staged = mode == 5 || mode == 7;
   if (staged) mode -= 4;
   if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
-  const bool direct_ok = head_dim == DIRECT_D && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
+  // (the kernel that brings pages straight into LDS knows neither a cap nor a sink)
+  const bool direct_ok = head_dim == DIRECT_D && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0 &&
+                         !(opt.softcap > 0.f) && opt.sink == nullptr;
   if (mode == 0) {
     // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
     // is read from LDS twice; they also halve the number of workgroups, so they need four of them for every
@@ -1187,7 +1226,7 @@ static int causal_entry(const void* q, const void* k_pages, const void* v_pages,
   }
 #define CAUSAL(GPV, RPV)                                                                                          \
   return launch_causal<GPV, RPV>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, \
-                                 n_seqs, max_tiles, out, n_heads, n_kv, head_dim, scale, window, stream)
+                                 n_seqs, max_tiles, out, n_heads, n_kv, head_dim, scale, window, opt, stream)
   if (direct_ok && !staged && mode != 2) {
     if (mode == 3)
       return launch_causal_direct<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
@@ -1205,10 +1244,12 @@ static int causal_entry(const void* q, const void* k_pages, const void* v_pages,
 DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                      int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                      const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
-                                     int n_kv, int head_dim, float scale, int window, int mode, hipStream_t stream) {
+                                     int n_kv, int head_dim, float scale, int window, int mode, float softcap,
+                                     const float* sink, hipStream_t stream) {
   ProjectedQ none = {};
   return causal_entry(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                      max_tiles, out, n_heads, n_kv, head_dim, scale, window, mode, none, stream);
+                      max_tiles, out, n_heads, n_kv, head_dim, scale, window, mode, none, stream,
+                      ScoreOptions{softcap, sink});
 }
 
 // Can the causal kernel take the queries from the fused projection itself (norm, rotation over `rot` features)?
@@ -1234,7 +1275,7 @@ DRYFT_API int dryft_attn_causal_projected_bf16(const void* qkv, int64_t qkv_stri
 static int launch_split(const void* q, const void* k_pages, const void* v_pages, const int* page_table, int max_pages,
                         const int* seq_slot, const int* cu_rows, const int* kv_len, int n_seqs, float* part_o,
                         float* part_ml, int n_splits, void* out, int n_heads, int n_kv, int head_dim, float scale,
-                        int window, FusedQKV fused, hipStream_t stream) {
+                        int window, FusedQKV fused, hipStream_t stream, ScoreOptions opt = {0.f, nullptr}) {
   if (n_seqs <= 0) return 0;
   if (!head_shape_ok(n_heads, n_kv, head_dim) || n_splits < 1 || n_splits > COMBINE_MAX_SPLITS) return -1;
   const int group = n_heads / n_kv, blocks = (group + 15) / 16;
@@ -1244,7 +1285,7 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
   hipLaunchKernelGGL((attn_split_kernel<KB, FULLV>), grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages, \
                      (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, part_o, part_ml,    \
                      n_heads, n_kv, head_dim, scale, window, n_splits, fused, (bf16_t*)k_pages, (bf16_t*)v_pages,       \
-                     (bf16_t*)out)
+                     (bf16_t*)out, opt)
   if (head_dim % 32 == 0) {
     DISPATCH_KB(head_dim / 32, LAUNCH_SPLIT(true));
   } else {
@@ -1255,7 +1296,7 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
   if (rc || n_splits == 1) return rc;
 #define COMBINE(HELD)                                                                                              \
   hipLaunchKernelGGL(attn_combine_kernel<HELD>, dim3(n_seqs, n_heads), dim3(COMBINE_THREADS), 0, stream, part_o,   \
-                     part_ml, seq_slot, cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits)
+                     part_ml, seq_slot, cu_rows, (bf16_t*)out, n_heads, head_dim, n_splits, opt.sink)
   if (n_splits <= 4) COMBINE(4);
   else if (n_splits <= 8) COMBINE(8);
   else if (n_splits <= 16) COMBINE(16);
@@ -1267,10 +1308,11 @@ static int launch_split(const void* q, const void* k_pages, const void* v_pages,
 DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                     int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
                                     int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
-                                    int n_kv, int head_dim, float scale, int window, hipStream_t stream) {
+                                    int n_kv, int head_dim, float scale, int window, float softcap, const float* sink,
+                                    hipStream_t stream) {
   FusedQKV none = {};
   return launch_split(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, n_seqs, part_o, part_ml,
-                      n_splits, out, n_heads, n_kv, head_dim, scale, window, none, stream);
+                      n_splits, out, n_heads, n_kv, head_dim, scale, window, none, stream, ScoreOptions{softcap, sink});
 }
 
 // The same with the work of the norm/rotation/append kernel folded in: `qkv` is the fused projection's output

@@ -101,7 +101,8 @@ class GQAAttention(Mixer):
                       self.value_dim if self.value_dim != self.head_dim else None)
 
     def kernel_modules(self, dtype):
-        return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ())
+        return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ()) + \
+            (("activation",) if self.output_gate else ())
 
     def _forward_general(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
         """Every option, in float arithmetic on the kernel that takes one (row, head) a workgroup."""
@@ -121,9 +122,30 @@ class GQAAttention(Mixer):
         q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
         ops.rope_pairs_kv(proj, 0, self.q_dim, self.q_dim + self.kv_dim, cos, sin, rot, ctx.row_slot, ctx.row_pos, q,
                           line.k, line.v, line.page_table, writes_cache, H, G, D, Dv)
-        out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
-        ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
-                      self.window or 0, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights)
+        # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16);
+        # float32, and the other sizes, on the kernel that takes one (row, head) a workgroup in float arithmetic
+        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0
+        window = self.window or 0
+        if matrix_cores and ctx.max_q_len == 1:
+            out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
+            splits = self.decode_splits(ctx.n_seqs, ctx.max_kv_len)
+            part_o = torch.empty((ctx.n_seqs, H, splits, D), dtype=torch.float32, device=h.device)
+            part_ml = torch.empty((ctx.n_seqs, H, splits, 2), dtype=torch.float32, device=h.device)
+            ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len, ctx.n_seqs,
+                                part_o, part_ml, splits, out, H, G, D, self.scale, window, softcap=self.softcap,
+                                sink=self.sink)
+        elif matrix_cores:
+            # the tiled kernel never visits the rows of sequences that sit out; they must hold something finite
+            out = ctx.kept_zeros((rows, H, Dv), h.dtype) if ctx.some_sit_out() else \
+                torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
+            tile_cu, max_tiles = ctx.tiles(ops.ATTN_ROW_TILE)
+            ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, tile_cu, ctx.seq_start,
+                                 ctx.n_seqs, max_tiles, out, H, G, D, self.scale, window, softcap=self.softcap,
+                                 sink=self.sink)
+        else:
+            out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
+            ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
+                          window, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights)
         out = out.view(rows, self.o_dim)
         if self.output_gate:
             gated = torch.empty_like(out)
