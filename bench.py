@@ -41,9 +41,99 @@ def prefill_flops(engine, tokens: int) -> float:
     return engine.model.step_flops([(0, tokens)], 1)
 
 
+def measure(engine, prompt_len: int, batch: int, steps: int, warmup: int, seed: int = 0) -> dict:
+    """Prefill of one prompt and decoding at one batch size through the generation loop, each with the fraction of
+    its roofline: the step's floating-point operations over the bf16 matrix-core peak, the bytes a decoding step has
+    to read over the HBM peak."""
+    import numpy as np
+    import torch
+
+    rng = np.random.default_rng(seed)
+    vocab = engine.model.plan.vocab_size
+
+    def prompts(b):
+        return [[int(t) for t in rng.integers(0, vocab, size=prompt_len)] for _ in range(b)]
+
+    best = None
+    for _ in range(3):                                     # the first run warms libraries up
+        slots = engine.acquire(1)
+        p = prompts(1)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.start(slots, p, 0)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.release(slots)
+        best = dt if best is None else min(best, dt)
+    flops = engine.model.step_flops([(0, prompt_len)], 1)
+    stream = engine.generate(prompts(batch), warmup + steps + 1)
+    try:
+        for _ in range(warmup + 1):
+            next(stream)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            next(stream)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    finally:
+        stream.close()
+    need = decode_bytes(engine, batch, prompt_len + warmup + (steps + 1) / 2.0)
+    return {"weights_gb": round(engine.model.streamed_weight_bytes() / 1e9, 3),
+            "prefill_tok_s": round(prompt_len / best, 1), "prefill_ms": round(best * 1e3, 3),
+            "prefill_tflop": round(flops / 1e12, 3), "prefill_frac": round(flops / best / PEAK_FLOPS["bf16"], 4),
+            "decode_tok_s": round(batch * steps / dt, 1), "decode_ms": round(dt / steps * 1e3, 4),
+            "decode_gbytes": round(need / 1e9, 4), "decode_frac": round(need / (dt / steps) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
+def compare_designs(args) -> int:
+    """``--design piralix``: Piralix at a few sizes with the widths of real models' layers beside a Qwen3 of the same
+    width, heads, feed-forward and vocabulary whose number of layers gives it the same weight bytes; random weights,
+    bfloat16, one prompt of ``--prompt-len`` tokens and ``--batch`` sequences decoding. One JSON line."""
+    import torch
+
+    from dryft_amd import Engine
+    from dryft_amd.models import load_preset
+
+    sizes = []
+    for name in args.sizes.split(","):
+        raw = load_preset(name)
+        kw = dict(seed=args.seed, dtype="bfloat16", max_batch=args.batch, max_len=args.prompt_len + 2 * (args.steps + args.warmup) + 64,
+                  use_graph=not args.no_graph)
+        engine = Engine(config=raw, **kw)
+        new = measure(engine, args.prompt_len, args.batch, args.steps, args.warmup, args.seed)
+        bytes_new = engine.model.streamed_weight_bytes()
+        del engine
+        torch.cuda.empty_cache()
+        att = next(l for l in raw["layers"] if l["type"] == "attention")
+        twin = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "num_hidden_layers": 1,
+                "hidden_size": raw["width"], "num_attention_heads": att["mixer"]["heads"],
+                "num_key_value_heads": att["mixer"]["kv_heads"], "head_dim": att["mixer"]["dim"],
+                "intermediate_size": att["mlp"]["ff"], "vocab_size": raw["vocab"], "rope_theta": 1000000.0,
+                "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "hidden_act": "silu", "attention_bias": False}
+        h, d = raw["width"], att["mixer"]["dim"]
+        per_layer = 2 * (h * d * (2 * att["mixer"]["heads"] + 2 * att["mixer"]["kv_heads"]) + 3 * h * att["mlp"]["ff"])
+        twin["num_hidden_layers"] = max(1, round((bytes_new - 2 * raw["vocab"] * h) / per_layer))
+        engine = Engine(config=twin, **kw)
+        old = measure(engine, args.prompt_len, args.batch, args.steps, args.warmup, args.seed)
+        del engine
+        torch.cuda.empty_cache()
+        sizes.append({"preset": name, "width": h, "piralix_layer_runs": len(raw["layers"]) + (raw["loop"]["times"] - 1) *
+                      (raw["loop"]["stop"] - raw["loop"]["start"]), "qwen3_layers": twin["num_hidden_layers"],
+                      "piralix": new, "qwen3": old})
+    print(json.dumps({"metric": "prefill and decode of Piralix beside Qwen3 of equal width and weight bytes",
+                      "dtype": "bf16", "data": "synthetic (random weights, uniform random token ids)",
+                      "prompt_len": args.prompt_len, "batch": args.batch, "steps": args.steps, "warmup": args.warmup,
+                      "graph": not args.no_graph, "sizes": sizes}))
+    return 0
+
+
 def main() -> int:
     global PROMPT, SLOT
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", default=None, choices=["piralix"],
+                    help="instead of the default workload: that design beside Qwen3 at equal size (one JSON line)")
+    ap.add_argument("--sizes", default="piralix-w1024,piralix-w2048,piralix-w2560", help="presets for --design")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -63,6 +153,8 @@ def main() -> int:
     args = ap.parse_args()
     PROMPT = args.prompt_len
     SLOT = args.slot_len or max(SLOT, 2 * PROMPT)
+    if args.design:
+        return compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")
         return 2

@@ -188,3 +188,293 @@ DRYFT_API int dryft_mlstm_out(const float* o_raw, const void* proj, int64_t proj
                        g_col, w, row_slot, (bf16_t*)out, n_heads, v_dim, eps);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// The same recurrence for steps of many rows in bfloat16, a chunk of 64 tokens at a time on the matrix cores.
+// The running maximum obeys m_t = b_t + M_t with b_t the sum of the chunk's log forget gates up to t and
+// M_t = max(m_0, max_(s<=t) c_s), c_s = i_s - b_s, so every weight of the chunk is known before any product:
+//
+//   o_t   = [ e_t (q_t . S_0) + sum_(s<=t) P_ts v_s ] / (max(|e_t (q_t . n_0) + sum_(s<=t) P_ts|, exp(-m_t)) + 1e-6)
+//   P_ts  = (q_t . k_s) exp(c_s - M_t),   e_t = exp(m_0 - M_t)                       (both at most 1)
+//   S_L   = exp(m_0 - M_L) S_0 + sum_s exp(c_s - M_L) k_s v_s^T,   n_L likewise,   m_L = b_L + M_L
+//
+// which is the token-by-token recurrence written out (same m_t, same weights). Gates, weights, maxima,
+// normalisers, the decay of the state and the state itself are float32; the operands of the four products
+// (q k^T, P v, q S_0, k^T v) are bfloat16 with float32 accumulation, as in attention. A workgroup of four waves
+// owns one (sequence, head, 64 value columns) and walks the sequence's chunks in order with S^T in its
+// accumulators: C[m = value column][n = key feature]. Operand layout of the 16x16x32 instruction as everywhere in
+// this library: A lane (c, g) holds row c, k = 8g..8g+7; B likewise for column c; C lane holds rows 4g..4g+3 of
+// column c. Products are arranged so that tokens (or key features) are the n index and operands come row-wise
+// from LDS: scores^T = K Q^T, O^T = V^T P^T + S_0^T Q^T, dS^T = V^T K'. V^T and K'^T = (w_s k_s)^T are staged with the
+// chunk's positions in the order in which the scores leave them in a lane (value_column).
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16((a), (b), (c), 0, 0, 0)
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define CH_L 64                 // tokens a chunk
+#define CH_VS 64                // value columns a workgroup
+#define CH_PAD 8
+#define CH_MAX_DT 4             // tiles of 16 key features a wave may own: D <= 256
+
+template <int KB>               // KB = ceil(D / 32)
+__global__ __launch_bounds__(256) void mlstm_chunks_kernel(
+    const bf16_t* __restrict__ proj, int64_t proj_stride, int q_col, int k_col, int v_col,
+    const float* __restrict__ gates, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
+    const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
+    float* __restrict__ state_s, float* __restrict__ state_n, float* __restrict__ state_m,
+    float* __restrict__ o_raw, int n_heads, int dim, int v_dim, float q_scale, int write_state) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  constexpr int DP = 32 * KB;                                   // key features, padded with zeros
+  constexpr int KS = DP + CH_PAD, TS = CH_L + CH_PAD;           // row strides in LDS
+  constexpr int DT = (DP / 16 + 3) / 4;                         // key-feature tiles a wave owns
+  const int seq = blockIdx.x, head = blockIdx.y, v0 = blockIdx.z * CH_VS;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int row0 = cu_rows[seq], n_tok = q_len[seq];
+  bf16_t* k_s = (bf16_t*)lds_raw;                               // [64][KS]      keys, row-wise
+  bf16_t* kw_t = k_s + CH_L * KS;                               // [DP][TS]      (w_s k_s)^T, positions permuted
+  bf16_t* v_t = kw_t + DP * TS;                                 // [64][TS]      V^T, positions permuted
+  bf16_t* s_t = v_t + CH_VS * TS;                               // [64][KS]      S_0^T rounded
+  float* n_s = (float*)(s_t + CH_VS * KS);                      // [DP]
+  float* g_M = n_s + DP;                                        // [64] M_t
+  float* g_c = g_M + CH_L;                                      // [64] c_s
+  float* g_b = g_c + CH_L;                                      // [64] b_t
+  float* g_x = g_b + CH_L;                                      // [4]  M_L, b_L
+  const int64_t sh = (int64_t)slot * n_heads + head;
+  float* S = state_s + sh * dim * v_dim;
+  float* N = state_n + sh * dim;
+  // the state: S^T tiles [value tile vt][own key-feature tile j], d-tile index = wave + 4 j
+  f32x4 acc_s[4][DT];
+#pragma unroll
+  for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+    for (int j = 0; j < DT; ++j) {
+      const int d = 16 * (wave + 4 * j) + c;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int v = v0 + 16 * vt + 4 * g + i;
+        acc_s[vt][j][i] = (d < dim && v < v_dim) ? S[(int64_t)d * v_dim + v] : 0.f;
+      }
+    }
+  for (int d = threadIdx.x; d < DP; d += blockDim.x) n_s[d] = d < dim ? N[d] : 0.f;
+  float m0 = state_m[sh];
+  for (int t0 = 0; t0 < n_tok; t0 += CH_L) {
+    const int nt = min(CH_L, n_tok - t0);
+    __syncthreads();                                            // the chunk before is done with every buffer
+    // S_0^T rounded, for the read-out of this chunk
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+      for (int j = 0; j < DT; ++j) {
+        const int d = 16 * (wave + 4 * j) + c;
+        if (d < DP) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s_t[(16 * vt + 4 * g + i) * KS + d] = float_to_bf16(acc_s[vt][j][i]);
+        }
+      }
+    // the chunk's gates: one lane a token
+    if (wave == 0) {
+      const bool live = lane < nt;
+      const float* gp = gates + (int64_t)(row0 + t0 + (live ? lane : 0)) * 2 * n_heads;
+      const float gi = cap * tanhf((gp[head] + bias_i[head]) / cap);
+      float b = live ? log_sigmoid(cap * tanhf((gp[n_heads + head] + bias_f[head]) / cap)) : 0.f;
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {                      // inclusive sum over the lanes before
+        const float up = __shfl_up(b, o, WAVE);
+        if (lane >= o) b += up;
+      }
+      const float cs = live ? gi - b : -INFINITY;
+      float M = fmaxf(cs, lane == 0 ? m0 : -INFINITY);
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float up = __shfl_up(M, o, WAVE);
+        if (lane >= o) M = fmaxf(M, up);
+      }
+      g_M[lane] = M;
+      g_c[lane] = cs;
+      g_b[lane] = b;
+      if (lane == nt - 1) { g_x[0] = M; g_x[1] = b; }
+    }
+    __syncthreads();
+    const float M_L = g_x[0], b_L = g_x[1];
+    // stage the chunk: K row-wise; (w_s k_s)^T and V^T with the positions in the lanes' order
+    for (int e = threadIdx.x; e < CH_L * (DP / 8); e += blockDim.x) {
+      const int s = e / (DP / 8), d = 8 * (e % (DP / 8));
+      float kv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (s < nt && d < dim)                                    // dim is a multiple of 8 (the host checks)
+        load8_as_float(proj + (int64_t)(row0 + t0 + s) * proj_stride + k_col + (int64_t)head * dim + d, kv);
+      store8_from_float(k_s + s * KS + d, kv);
+      const float w = s < nt ? expf(g_c[s] - M_L) : 0.f;
+      const int col = value_column(s);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) kw_t[(d + j) * TS + col] = float_to_bf16(w * kv[j]);
+    }
+    for (int e = threadIdx.x; e < CH_L * (CH_VS / 8); e += blockDim.x) {
+      const int s = e / (CH_VS / 8), v = 8 * (e % (CH_VS / 8));
+      float vv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (s < nt && v0 + v < v_dim)                             // v_dim is a multiple of 8
+        load8_as_float(proj + (int64_t)(row0 + t0 + s) * proj_stride + v_col + (int64_t)head * v_dim + v0 + v, vv);
+      const int col = value_column(s);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v_t[(v + j) * TS + col] = float_to_bf16(vv[j]);
+    }
+    // this wave's 16 tokens: the queries stay in registers
+    const int t = 16 * wave + c;                                // the lane's token of the chunk
+    const bool t_live = t < nt;
+    bf16x8 q[KB];
+    float qn = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int d = 32 * kb + 8 * g;
+      float qv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (t_live && d < dim)
+        load8_as_float(proj + (int64_t)(row0 + t0 + t) * proj_stride + q_col + (int64_t)head * dim + d, qv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        q[kb][j] = (__bf16)qv[j];
+        qn += qv[j] * n_s[d + j];
+      }
+    }
+    qn += __shfl_xor(qn, 16, WAVE);
+    qn += __shfl_xor(qn, 32, WAVE);
+    __syncthreads();                                            // the chunk is staged
+    const float M_t = t_live ? g_M[t] : 0.f;
+    const float e_t = t_live ? expf(m0 - M_t) * q_scale : 0.f;
+    f32x4 acc_o[4];
+    if (16 * wave < nt) {
+      // q S_0
+#pragma unroll
+      for (int vt = 0; vt < 4; ++vt) {
+        acc_o[vt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          acc_o[vt] = MFMA16(*(const bf16x8*)(s_t + (16 * vt + c) * KS + 32 * kb + 8 * g), q[kb], acc_o[vt]);
+        acc_o[vt] *= e_t;
+      }
+      // the chunk's own tokens up to each row
+      float row_sum = 0.f;
+      bf16x8 p[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) p[h][j] = (__bf16)0.f;
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        if (st > wave) continue;                                // positions after all of the wave's rows
+        f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          sc = MFMA16(*(const bf16x8*)(k_s + (16 * st + c) * KS + 32 * kb + 8 * g), q[kb], sc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int s = 16 * st + 4 * g + i;
+          const float pw = (t_live && s <= t) ? sc[i] * q_scale * expf(g_c[s] - M_t) : 0.f;
+          row_sum += pw;
+          p[st / 2][4 * (st & 1) + i] = (__bf16)pw;
+        }
+      }
+      row_sum += __shfl_xor(row_sum, 16, WAVE);
+      row_sum += __shfl_xor(row_sum, 32, WAVE);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        if (32 * h > 16 * wave + 15) continue;                  // a block of positions after all of the wave's rows
+#pragma unroll
+        for (int vt = 0; vt < 4; ++vt)
+          acc_o[vt] = MFMA16(*(const bf16x8*)(v_t + (16 * vt + c) * TS + 32 * h + 8 * g), p[h], acc_o[vt]);
+      }
+      if (t_live) {
+        const float m_t = g_b[t] + M_t;
+        const float den = fmaxf(fabsf(e_t * qn + row_sum), expf(-m_t)) + 1e-6f;
+        float* o = o_raw + ((int64_t)(row0 + t0 + t) * n_heads + head) * v_dim + v0;
+#pragma unroll
+        for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int v = 16 * vt + 4 * g + i;
+            if (v0 + v < v_dim) o[v] = acc_o[vt][i] / den;
+          }
+      }
+    }
+    // the state after the chunk
+    const float decay = expf(m0 - M_L);
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+      for (int j = 0; j < DT; ++j) {
+        if (16 * (wave + 4 * j) >= DP) continue;
+        acc_s[vt][j] *= decay;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          acc_s[vt][j] = MFMA16(*(const bf16x8*)(v_t + (16 * vt + c) * TS + 32 * h + 8 * g),
+                                *(const bf16x8*)(kw_t + (16 * (wave + 4 * j) + c) * TS + 32 * h + 8 * g), acc_s[vt][j]);
+      }
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+      float a = decay * n_s[d];
+      for (int s = 0; s < nt; ++s) a += expf(g_c[s] - M_L) * bf16_to_float(k_s[s * KS + d]);
+      n_s[d] = a;
+    }
+    m0 = b_L + M_L;
+  }
+  if (!write_state) return;
+#pragma unroll
+  for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+    for (int j = 0; j < DT; ++j) {
+      const int d = 16 * (wave + 4 * j) + c;
+      if (d >= dim) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int v = v0 + 16 * vt + 4 * g + i;
+        if (v < v_dim) S[(int64_t)d * v_dim + v] = acc_s[vt][j][i];
+      }
+    }
+  if (blockIdx.z == 0) {
+    __syncthreads();
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) N[d] = n_s[d];
+    if (threadIdx.x == 0) state_m[sh] = m0;
+  }
+}
+
+// Does the chunked kernel take these sizes? (16-byte pieces of rows; key width up to 256.)
+DRYFT_API int dryft_mlstm_chunks_takes(int dim, int v_dim, int q_col, int k_col, int v_col, int64_t proj_stride) {
+  return dim > 0 && dim <= 64 * CH_MAX_DT && dim % 8 == 0 && v_dim % 8 == 0 && q_col % 8 == 0 && k_col % 8 == 0 &&
+         v_col % 8 == 0 && proj_stride % 8 == 0;
+}
+
+DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_col, int k_col, int v_col,
+                                 const float* gates, const float* bias_i, const float* bias_f, float cap,
+                                 const int* seq_slot, const int* cu_rows, const int* q_len, int n_seqs, float* state_s,
+                                 float* state_n, float* state_m, float* o_raw, int n_heads, int dim, int v_dim,
+                                 float q_scale, int write_state, hipStream_t stream) {
+  if (n_seqs <= 0) return 0;
+  if (!dryft_mlstm_chunks_takes(dim, v_dim, q_col, k_col, v_col, proj_stride) || ((uintptr_t)proj & 15) || !(cap > 0.f))
+    return -1;
+  const int kb = (dim + 31) / 32, dp = 32 * kb;
+  const size_t lds = (size_t)(2 * CH_L * (dp + CH_PAD) + dp * (CH_L + CH_PAD) + CH_VS * (CH_L + CH_PAD)) * 2 +
+                     (size_t)(dp + 3 * CH_L + 4) * sizeof(float);
+  dim3 grid(n_seqs, n_heads, (v_dim + CH_VS - 1) / CH_VS), block(256);
+#define MC(KBV)                                                                                                      \
+  {                                                                                                                  \
+    auto kernel = mlstm_chunks_kernel<KBV>;                                                                          \
+    if (lds > 64 * 1024 &&                                                                                           \
+        hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return -1;                                                                                                     \
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)proj, proj_stride, q_col, k_col, v_col, gates, \
+                       bias_i, bias_f, cap, seq_slot, cu_rows, q_len, state_s, state_n, state_m, o_raw, n_heads, dim,  \
+                       v_dim, q_scale, write_state);                                                                 \
+  }
+  switch (kb) {
+    case 1: MC(1); break;
+    case 2: MC(2); break;
+    case 3: MC(3); break;
+    case 4: MC(4); break;
+    case 5: MC(5); break;
+    case 6: MC(6); break;
+    case 7: MC(7); break;
+    case 8: MC(8); break;
+    default: return -1;
+  }
+#undef MC
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(const void* __restrict
                                                           const void* __restrict__ w, int w_f32,
                                                           float* __restrict__ x_out, T* __restrict__ y, int width,
                                                           float eps) {
-  extern __shared__ float held[];
+  extern __shared__ __attribute__((aligned(16))) float held[];
   __shared__ float scratch[16];
   const int64_t base = (int64_t)blockIdx.x * width;
   float inv_d = 1.f;
@@ -231,6 +231,92 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(const void* __restrict
     store_from_float(y + base + i, held[i] * inv * load_vector(w, i, w_f32));
 }
 
+// The same for rows whose width is a multiple of 8 with 16-byte aligned operands: a thread owns runs of 8
+// contiguous values, moves them with 16-byte loads and stores, and asks for four partial sums at a time, so that a
+// row of a decoding step (latency, not bandwidth) costs a few trips to memory instead of one per value and part.
+template <typename T, typename D>
+__global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __restrict__ x_in, int x_kind,
+                                                              const D* __restrict__ delta, int n_partials,
+                                                              int64_t partial_stride, const void* __restrict__ wb,
+                                                              int wb_f32, const T* __restrict__ extra,
+                                                              const void* __restrict__ vec, int vec_f32,
+                                                              const void* __restrict__ w, int w_f32,
+                                                              float* __restrict__ x_out, T* __restrict__ y, int width,
+                                                              float eps) {
+  extern __shared__ __attribute__((aligned(16))) float held[];
+  __shared__ float scratch[16];
+  const int64_t base = (int64_t)blockIdx.x * width;
+  float inv_d = 1.f;
+  if (n_partials > 0) {
+    float ss = 0.f;
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+      float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      int p = 0;
+      for (; p + 4 <= n_partials; p += 4) {               // four loads in flight; added in the order 0, 1, ...
+        float t[4][8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) load8_as_float(delta + (p + u) * partial_stride + base + i, t[u]);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) d[j] += t[u][j];
+      }
+      for (; p < n_partials; ++p) {
+        float t[8];
+        load8_as_float(delta + p * partial_stride + base + i, t);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) d[j] += t[j];
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += d[j] * d[j];
+      store8_from_float(held + i, d);
+    }
+    if (wb != nullptr) inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, t[8];
+    if (x_kind == 2) load8_as_float((const float*)x_in + base + i, v);
+    else if (x_kind == 1) load8_as_float((const T*)x_in + base + i, v);
+    if (n_partials > 0) {
+      load8_as_float(held + i, t);
+      if (wb != nullptr) {
+        float wv[8];
+        if (wb_f32) load8_as_float((const float*)wb + i, wv); else load8_as_float((const bf16_t*)wb + i, wv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += t[j] * inv_d * wv[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] += t[j];
+      }
+    }
+    if (extra != nullptr) {
+      load8_as_float(extra + base + i, t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += t[j];
+    }
+    if (vec != nullptr) {
+      if (vec_f32) load8_as_float((const float*)vec + i, t); else load8_as_float((const bf16_t*)vec + i, t);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += t[j];
+    }
+    store8_from_float(held + i, v);
+    if (x_out != nullptr) store8_from_float(x_out + base + i, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+  }
+  if (y == nullptr) return;
+  const float inv = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+    float v[8], wv[8];
+    load8_as_float(held + i, v);
+    if (w_f32) load8_as_float((const float*)w + i, wv); else load8_as_float((const bf16_t*)w + i, wv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] *= inv * wv[j];
+    store8_from_float(y + base + i, v);
+  }
+}
+
 #define STREAM_NORM_MAX_WIDTH 16384   // 64 KiB of LDS a row
 
 // x_kind: 0 = no stream yet, 1 = the stream in the activation dtype, 2 = float32.
@@ -248,6 +334,19 @@ DRYFT_API int dryft_stream_norm(const void* x_in, int x_kind, const void* delta,
   hipLaunchKernelGGL((stream_norm_kernel<TT, DD>), grid, block, lds, stream, x_in, x_kind, (const DD*)delta,        \
                      n_partials, partial_stride, wb, wb_f32, (const TT*)extra, vec, vec_f32, w, w_f32, x_out,       \
                      (TT*)y, width, eps)
+#define SNV(TT, DD)                                                                                                  \
+  hipLaunchKernelGGL((stream_norm_vec_kernel<TT, DD>), grid, block, lds, stream, x_in, x_kind, (const DD*)delta,    \
+                     n_partials, partial_stride, wb, wb_f32, (const TT*)extra, vec, vec_f32, w, w_f32, x_out,       \
+                     (TT*)y, width, eps)
+  const bool aligned = (((uintptr_t)x_in | (uintptr_t)delta | (uintptr_t)wb | (uintptr_t)extra | (uintptr_t)vec |
+                         (uintptr_t)w | (uintptr_t)x_out | (uintptr_t)y) & 15) == 0 && partial_stride % 4 == 0;
+  if (width % 8 == 0 && aligned) {
+    if (is_f32) SNV(float, float);
+    else if (delta_kind == 2) SNV(bf16_t, float);
+    else SNV(bf16_t, bf16_t);
+    return DRYFT_LAUNCH_CHECK();
+  }
+#undef SNV
   if (is_f32) SN(float, float);
   else if (delta_kind == 2) SN(bf16_t, float);
   else SN(bf16_t, bf16_t);

@@ -29,9 +29,15 @@ _SIGNATURES = {
                    "dryft_sigmoid_gate": [_P, _L, _P, _L, _P, _I, _I, _I, _P]},
     "mlstm": {"dryft_mlstm_steps": [_P, _L, _I, _I, _I, _P, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F,
                                     _I, _I, _P],
+              "dryft_mlstm_chunks_takes": [_I, _I, _I, _I, _I, _L],
+              "dryft_mlstm_chunks": [_P, _L, _I, _I, _I, _P, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F,
+                                     _I, _P],
               "dryft_mlstm_out": [_P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "rglru": {"dryft_rglru_gates": [_P, _L, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _P, _P, _I, _I,
                                     _I, _I, _P],
+              "dryft_rglru_tile_rows": [],
+              "dryft_rglru_scan_tiles": [_P, _P, _P, _L, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I,
+                                         _I, _P],
               "dryft_rglru_scan": [_P, _P, _L, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _P]},
     "rope_kv": {"dryft_qk_norm_rope_kv": [_P, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                           _I, _I, _I, _I, _I, _P],
@@ -1068,9 +1074,15 @@ def _seq_facts(seq_slot, cu_rows, q_len, n_seqs: int) -> None:
 MLSTM_MAX_DIM = 256
 
 
+def mlstm_chunks_takes(proj, q_col: int, k_col: int, v_col: int, dim: int, v_dim: int) -> bool:
+    """Does the chunked matrix-core form of ``mlstm_steps`` take this projection? (bfloat16, 16-byte pieces.)"""
+    return proj.dtype == torch.bfloat16 and proj.data_ptr() % 16 == 0 and bool(
+        _fn("mlstm", "dryft_mlstm_chunks_takes")(dim, v_dim, q_col, k_col, v_col, proj.stride(0)))
+
+
 def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f, cap: float, seq_slot, cu_rows, q_len,
                 n_seqs: int, state_s, state_n, state_m, o_raw, n_heads: int, dim: int, v_dim: int, q_scale: float,
-                write_state: bool) -> None:
+                write_state: bool, chunked: bool = False) -> None:
     """The matrix-memory recurrence over each sequence's rows of the step, in order; ``o_raw`` (float32
     ``[rows, heads, v_dim]``) receives each token's read-out divided by its normaliser. ``gates`` are the float32
     projections ``[rows, 2 * heads]`` (input gates, then forget gates) before bias, cap and log-sigmoid. The states
@@ -1100,6 +1112,15 @@ def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f,
     _gpu(o_raw, "o_raw", torch.float32)
     if not (o_raw.is_contiguous() and o_raw.numel() == rows * n_heads * v_dim):
         raise KernelError("mlstm_steps: o_raw must be float32 [rows, heads, v_dim]")
+    if chunked:
+        # the same recurrence a chunk of 64 tokens at a time on the matrix cores (steps of many rows, bfloat16)
+        if not mlstm_chunks_takes(proj, q_col, k_col, v_col, dim, v_dim):
+            raise KernelError("mlstm_steps: the chunked kernel does not take these sizes")
+        _check(_fn("mlstm", "dryft_mlstm_chunks")(
+            _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),
+            _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs, _ptr(state_s), _ptr(state_n), _ptr(state_m),
+            _ptr(o_raw), n_heads, dim, v_dim, float(q_scale), int(bool(write_state)), _stream()), "mlstm_chunks")
+        return
     _check(_fn("mlstm", "dryft_mlstm_steps")(
         _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),
         _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs, _ptr(state_s), _ptr(state_n), _ptr(state_m), _ptr(o_raw),
@@ -1197,3 +1218,44 @@ def rglru_scan(coef, proj, x_col: int, y_col: int, x_bias, y_bias, taps: int, se
         _ptr(coef), _ptr(proj), proj.stride(0), x_col, y_col, _ptr(x_bias), _ptr(y_bias), taps, _ptr(seq_slot),
         _ptr(cu_rows), _ptr(q_len), _ptr(row_slot), n_seqs, _ptr(state), _ptr(tail) if taps > 1 else 0, _ptr(out), rows,
         width, int(bool(write_state)), _float_flag(proj, "proj"), _stream()), "rglru_scan")
+
+
+RGLRU_TILE = 64         # tokens of a sequence that one workgroup of the tiled walk takes (``ctx.tiles``)
+
+
+def rglru_scan_tiles(coef, proj, x_col: int, y_col: int, x_bias, y_bias, taps: int, seq_slot, cu_rows, q_len, tile_cu,
+                     max_tiles: int, n_seqs: int, state, tail, out, width: int, write_state: bool) -> None:
+    """``rglru_scan`` for steps of many rows per sequence: the walk cut into tiles of ``RGLRU_TILE`` tokens (their
+    prefix sums per sequence in ``tile_cu``, at most ``max_tiles`` in all) that run side by side. ``out``'s rows of
+    sequences that sit out are not written."""
+    if _fn("rglru", "dryft_rglru_tile_rows")() != RGLRU_TILE:
+        raise KernelError("rglru_scan_tiles: the library was built for another tile")
+    _gpu(proj, "proj")
+    rows = proj.shape[0]
+    _gpu(coef, "coef", torch.float32)
+    if not (tuple(coef.shape) == (rows, 2, width) and coef.is_contiguous()):
+        raise KernelError(f"coef: must be contiguous float32 [{rows}, 2, {width}]")
+    if not (proj.stride(1) == 1 and min(x_col, y_col) >= 0 and max(x_col, y_col) + width <= proj.shape[1]):
+        raise KernelError("rglru_scan_tiles: a branch lies outside the projection's columns")
+    _f32_vector(x_bias, "x_bias", width)
+    _f32_vector(y_bias, "y_bias", width)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(tile_cu, "tile_cu", torch.int32)
+    if not (tile_cu.is_contiguous() and tile_cu.numel() >= n_seqs + 1):
+        raise KernelError(f"tile_cu: needs {n_seqs + 1} contiguous entries")
+    _gpu(state, "state", torch.float32)
+    if not (state.dim() == 2 and state.shape[1] == width and state.is_contiguous()):
+        raise KernelError(f"state: must be contiguous float32 [slots, {width}]")
+    if taps > 1:
+        _gpu(tail, "tail", torch.float32)
+        if not (tuple(tail.shape) == (state.shape[0], taps - 1, width) and tail.is_contiguous()):
+            raise KernelError(f"tail: must be contiguous float32 [slots, {taps - 1}, {width}]")
+    _gpu(out, "out", proj.dtype)
+    if not (tuple(out.shape) == (rows, width) and out.is_contiguous()):
+        raise KernelError(f"out: must be contiguous [{rows}, {width}]")
+    ends = torch.empty((max(1, max_tiles), 2, width), dtype=torch.float32, device=proj.device)
+    _check(_fn("rglru", "dryft_rglru_scan_tiles")(
+        _ptr(coef), _ptr(ends), _ptr(proj), proj.stride(0), x_col, y_col, _ptr(x_bias), _ptr(y_bias), taps,
+        _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), _ptr(tile_cu), n_seqs, max_tiles, _ptr(state),
+        _ptr(tail) if taps > 1 else 0, _ptr(out), width, int(bool(write_state)), _float_flag(proj, "proj"), _stream()),
+        "rglru_scan_tiles")

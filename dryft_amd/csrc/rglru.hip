@@ -121,6 +121,135 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same walk for steps of many rows, cut into tiles of RG_TILE tokens so that a long prompt fills the chip.
+// S_t = a_t S_(t-1) + b_t is linear in S, so a tile is summed up by two numbers per channel, P = prod a and
+// Q = the tile's last S from S = 0. Three launches: every tile's (P, Q); per sequence and channel the state that
+// enters each tile, S <- P S + Q from tile to tile (a few dozen steps; this one also leaves the state and the
+// convolution's memory for the next step, and is the only one that touches them); every tile's own tokens from
+// the state that enters it. `tile_cu` are the prefix sums over the sequences of their tiles (a sequence that
+// sits out has none).
+#define RG_TILE 64
+
+__device__ __forceinline__ bool rg_locate(int tile, const int* __restrict__ tile_cu, int n_seqs, int& seq, int& in_seq) {
+  if (tile >= tile_cu[n_seqs]) return false;
+  int lo = 0, hi = n_seqs;                                      // last seq with tile_cu[seq] <= tile
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (tile_cu[mid] <= tile) lo = mid; else hi = mid;
+  }
+  while (lo + 1 < n_seqs && tile_cu[lo + 1] <= tile) ++lo;      // sequences without tiles share a start
+  seq = lo;
+  in_seq = tile - tile_cu[lo];
+  return true;
+}
+
+// ends: float32 [tiles, 2, width]: P, then Q.
+__global__ __launch_bounds__(256) void rglru_tile_ends_kernel(const float* __restrict__ coef,
+                                                              const int* __restrict__ cu_rows,
+                                                              const int* __restrict__ q_len,
+                                                              const int* __restrict__ tile_cu, int n_seqs,
+                                                              float* __restrict__ ends, int width) {
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  int seq, j;
+  if (!rg_locate(blockIdx.x, tile_cu, n_seqs, seq, j) || ch >= width) return;
+  const int t0 = j * RG_TILE, t1 = min(q_len[seq], t0 + RG_TILE);
+  float P = 1.f, Q = 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const float* c = coef + (int64_t)(cu_rows[seq] + t) * 2 * width;
+    P *= c[ch];
+    Q = c[ch] * Q + c[width + ch];
+  }
+  ends[((int64_t)blockIdx.x * 2) * width + ch] = P;
+  ends[((int64_t)blockIdx.x * 2 + 1) * width + ch] = Q;
+}
+
+// Turns ends[tile] = (P, Q) into ends[tile][0] = the state that enters the tile; leaves the step's last state.
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_carry_kernel(
+    float* __restrict__ ends, const T* __restrict__ proj, int64_t proj_stride, int x_col,
+    const float* __restrict__ x_bias, int taps, const int* __restrict__ seq_slot, const int* __restrict__ cu_rows,
+    const int* __restrict__ q_len, const int* __restrict__ tile_cu, float* __restrict__ state,
+    float* __restrict__ tail, int width, int write_state) {
+  const int seq = blockIdx.x, ch = blockIdx.y * blockDim.x + threadIdx.x;
+  if (ch >= width) return;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int row0 = cu_rows[seq], n_tok = q_len[seq];
+  float S = state[(int64_t)slot * width + ch];
+  for (int k = tile_cu[seq]; k < tile_cu[seq + 1]; ++k) {
+    float* e = ends + ((int64_t)k * 2) * width;
+    const float P = e[ch], Q = e[width + ch];
+    e[ch] = S;
+    S = P * S + Q;
+  }
+  if (!write_state) return;
+  state[(int64_t)slot * width + ch] = S;
+  const int keep = taps - 1;
+  float old[RG_MAX_TAPS];
+  float* tl = tail + (int64_t)slot * keep * width + ch;
+  for (int j = 0; j < keep; ++j) old[j] = tl[(int64_t)j * width];
+  for (int j = 0; j < keep; ++j) {
+    const int t = n_tok - keep + j;
+    float v;
+    if (t >= 0) v = load_as_float(proj + (int64_t)(row0 + t) * proj_stride + x_col + ch) + x_bias[ch];
+    else v = old[j + n_tok];
+    tl[(int64_t)j * width] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_apply_tiles_kernel(
+    const float* __restrict__ coef, const float* __restrict__ ends, const T* __restrict__ proj, int64_t proj_stride,
+    int y_col, const float* __restrict__ y_bias, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
+    const int* __restrict__ tile_cu, int n_seqs, T* __restrict__ out, int width) {
+  const int ch = blockIdx.y * blockDim.x + threadIdx.x;
+  int seq, j;
+  if (!rg_locate(blockIdx.x, tile_cu, n_seqs, seq, j) || ch >= width) return;
+  float S = ends[((int64_t)blockIdx.x * 2) * width + ch];
+  const float yb = y_bias[ch];
+  const int t0 = j * RG_TILE, t1 = min(q_len[seq], t0 + RG_TILE);
+  for (int t = t0; t < t1; ++t) {
+    const int64_t row = cu_rows[seq] + t;
+    const float* c = coef + row * 2 * width;
+    S = c[ch] * S + c[width + ch];
+    const float y = gelu_tanh(load_as_float(proj + row * proj_stride + y_col + ch) + yb);
+    store_from_float(out + row * width + ch, S * y);
+  }
+}
+
+DRYFT_API int dryft_rglru_tile_rows(void) { return RG_TILE; }
+
+// out must hold zeros (or anything finite) in the rows of sequences that sit out: no tile visits them.
+DRYFT_API int dryft_rglru_scan_tiles(const float* coef, float* ends, const void* proj, int64_t proj_stride, int x_col,
+                                     int y_col, const float* x_bias, const float* y_bias, int taps, const int* seq_slot,
+                                     const int* cu_rows, const int* q_len, const int* tile_cu, int n_seqs,
+                                     int max_tiles, float* state, float* tail, void* out, int width, int write_state,
+                                     int is_f32, hipStream_t stream) {
+  if (n_seqs <= 0 || max_tiles <= 0) return 0;
+  if (taps < 1 || taps > RG_MAX_TAPS) return -1;
+  const int cb = (width + 255) / 256;
+  if (cb > 65535) return -1;
+  hipLaunchKernelGGL(rglru_tile_ends_kernel, dim3(max_tiles, cb), dim3(256), 0, stream, coef, cu_rows, q_len, tile_cu,
+                     n_seqs, ends, width);
+  if (is_f32) {
+    hipLaunchKernelGGL(rglru_carry_kernel<float>, dim3(n_seqs, cb), dim3(256), 0, stream, ends, (const float*)proj,
+                       proj_stride, x_col, x_bias, taps, seq_slot, cu_rows, q_len, tile_cu, state, tail, width,
+                       write_state);
+    hipLaunchKernelGGL(rglru_apply_tiles_kernel<float>, dim3(max_tiles, cb), dim3(256), 0, stream, coef, ends,
+                       (const float*)proj, proj_stride, y_col, y_bias, cu_rows, q_len, tile_cu, n_seqs, (float*)out,
+                       width);
+  } else {
+    hipLaunchKernelGGL(rglru_carry_kernel<bf16_t>, dim3(n_seqs, cb), dim3(256), 0, stream, ends, (const bf16_t*)proj,
+                       proj_stride, x_col, x_bias, taps, seq_slot, cu_rows, q_len, tile_cu, state, tail, width,
+                       write_state);
+    hipLaunchKernelGGL(rglru_apply_tiles_kernel<bf16_t>, dim3(max_tiles, cb), dim3(256), 0, stream, coef, ends,
+                       (const bf16_t*)proj, proj_stride, y_col, y_bias, cu_rows, q_len, tile_cu, n_seqs, (bf16_t*)out,
+                       width);
+  }
+  return DRYFT_LAUNCH_CHECK();
+}
+
 DRYFT_API int dryft_rglru_gates(const void* proj, int64_t proj_stride, int x_col, const float* x_bias,
                                 const float* conv_w, const float* conv_b, int taps, const void* gate_a,
                                 const float* gate_a_bias, const void* gate_i, const float* gate_i_bias,

@@ -25,6 +25,9 @@ from .base import Mixer, StepContext, matrix
 from .linear import linear
 
 
+_CHUNKED_FROM = 8       # steps whose longest sequence brings more rows than this take the chunked matrix-memory kernel
+
+
 def _vector(n, init="normal"):
     return ((int(n),), VECTOR, init)
 
@@ -71,10 +74,14 @@ class MatrixMemory(Mixer):
         proj = linear(h, self.w_in)                                       # q | k | v | g, in the activation dtype
         gates = linear(h, self.w_gates, out_dtype=torch.float32)           # the gates stay float32 from here on
         o_raw = torch.empty((rows, self.n_heads, self.value_dim), dtype=torch.float32, device=h.device)
+        # steps of many rows in bfloat16: a chunk of tokens at a time on the matrix cores; single tokens, float32
+        # and sizes without 16-byte pieces: token by token in float arithmetic
+        chunked = ctx.max_q_len > _CHUNKED_FROM and \
+            ops.mlstm_chunks_takes(proj, 0, self.qk_dim, 2 * self.qk_dim, self.key_dim, self.value_dim)
         ops.mlstm_steps(proj, 0, self.qk_dim, 2 * self.qk_dim, gates, self.bias_i, self.bias_f, self.gate_cap,
                         ctx.seq_slot, ctx.cu_rows, ctx.q_len, ctx.n_seqs, line["memory"].state,
                         line["normaliser"].state, line["maximum"].state, o_raw, self.n_heads, self.key_dim,
-                        self.value_dim, self.key_dim ** -0.5, writes_cache)
+                        self.value_dim, self.key_dim ** -0.5, writes_cache, chunked=chunked)
         out = torch.empty((rows, self.v_dim), dtype=h.dtype, device=h.device)
         ops.mlstm_out(o_raw, proj, 2 * self.qk_dim + self.v_dim, self.out_norm, ctx.row_slot, out, self.n_heads,
                       self.value_dim, self.norm_eps)
@@ -132,6 +139,15 @@ class GatedLinearRecurrence(Mixer):
         ops.rglru_gates(proj, W, self.x_bias, self.conv, self.conv_bias, self.taps, self.gate_a, self.gate_a_bias,
                         self.gate_i, self.gate_i_bias, self.lam, self.decay_scale, ctx.row_slot, ctx.row_seq,
                         ctx.row_pos, ctx.seq_start, tail, coef, W, self.blocks)
+        if ctx.max_q_len > ops.RGLRU_TILE:
+            # a long prompt: its tiles of tokens side by side (rows of sequences that sit out are not visited)
+            out = ctx.kept_zeros((rows, W), h.dtype) if ctx.some_sit_out() else \
+                torch.empty((rows, W), dtype=h.dtype, device=h.device)
+            tile_cu, max_tiles = ctx.tiles(ops.RGLRU_TILE)
+            ops.rglru_scan_tiles(coef, proj, W, 0, self.x_bias, self.y_bias, self.taps, ctx.seq_slot, ctx.cu_rows,
+                                 ctx.q_len, tile_cu, max_tiles, ctx.n_seqs, line["state"].state, tail, out, W,
+                                 writes_cache)
+            return linear(out, self.w_o, allow_partials=True)
         out = torch.empty((rows, W), dtype=h.dtype, device=h.device)
         ops.rglru_scan(coef, proj, W, 0, self.x_bias, self.y_bias, self.taps, ctx.seq_slot, ctx.cu_rows, ctx.q_len,
                        ctx.row_slot, ctx.n_seqs, line["state"].state, tail, out, W, writes_cache)
