@@ -250,6 +250,89 @@ DRYFT_API int dryft_rglru_scan_tiles(const float* coef, float* ends, const void*
   return DRYFT_LAUNCH_CHECK();
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The gates on the matrix cores, for bfloat16 and blocks whose size is a multiple of 32. A workgroup takes up to
+// 64 rows of one block: it forms their convolution in float into LDS, then every wave multiplies its 16 rows with
+// the block's two gate matrices, 16 outputs at a time: C[m = output][n = row] = sum_k W[output][k] u[row][k], the
+// weights straight from memory (16 bytes a lane along k), u rounded to bfloat16 on its way out of LDS, the sums
+// float32. What follows the product (biases, sigmoids, the decay and its square root, the multiplication with the
+// unrounded u) is float arithmetic on the accumulators. With at most 16 rows in the step (decoding) the four
+// waves share those rows and deal the outputs among themselves, and among `gridDim.z` workgroups.
+#define MFMA16(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16((a), (b), (c), 0, 0, 0)
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+#define RG_MM_ROWS 64
+#define RG_MM_PAD 4
+
+__global__ __launch_bounds__(256) void rglru_gates_mfma_kernel(
+    const bf16_t* __restrict__ proj, int64_t proj_stride, int x_col, const float* __restrict__ x_bias,
+    const float* __restrict__ conv_w, const float* __restrict__ conv_b, int taps, const bf16_t* __restrict__ gate_a,
+    const float* __restrict__ gate_a_bias, const bf16_t* __restrict__ gate_i, const float* __restrict__ gate_i_bias,
+    const float* __restrict__ lam, float decay_scale, const int* __restrict__ row_slot,
+    const int* __restrict__ row_seq, const int* __restrict__ row_pos, const int* __restrict__ seq_start,
+    const float* __restrict__ tail, float* __restrict__ coef, int n_rows, int width, int block_size, int few) {
+  extern __shared__ __attribute__((aligned(16))) float u_s[];   // [rows of the workgroup][block_size + pad]
+  const int wg_rows = few ? 16 : RG_MM_ROWS;
+  const int r0 = blockIdx.x * wg_rows, b = blockIdx.y, ld = block_size + RG_MM_PAD;
+  const int rows = min(wg_rows, n_rows - r0);
+  for (int e = threadIdx.x; e < wg_rows * block_size; e += blockDim.x) {
+    const int rr = e / block_size, cc = e % block_size, ch = b * block_size + cc;
+    float u = 0.f;
+    if (rr < rows) {
+      const int64_t row = r0 + rr;
+      const int slot = row_slot[row];
+      if (slot >= 0) {
+        const int pos = row_pos[row], start = seq_start[row_seq[row]];
+        u = conv_b[ch];
+        for (int j = 0; j < taps; ++j) {
+          const int back = taps - 1 - j, p = pos - back;
+          float x;
+          if (p >= start) x = load_as_float(proj + (row - back) * proj_stride + x_col + ch) + x_bias[ch];
+          else x = tail[((int64_t)slot * (taps - 1) + (taps - 1 - start + p)) * width + ch];
+          u += conv_w[ch * taps + j] * x;
+        }
+      }
+    }
+    u_s[rr * ld + cc] = u;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int row_tile = few ? 0 : wave;                           // the wave's 16 rows within the workgroup's
+  if (16 * row_tile >= rows) return;
+  const int tiles = block_size / 16, kbs = block_size / 32;
+  const int first = few ? blockIdx.z * 4 + wave : 0, stride = few ? 4 * gridDim.z : 1;
+  const float* u_row = u_s + (16 * row_tile + c) * ld;
+  const int64_t row = r0 + 16 * row_tile + c;
+  const bool live = 16 * row_tile + c < rows && row_slot[min(row, (int64_t)n_rows - 1)] >= 0;
+  for (int ot = first; ot < tiles; ot += stride) {
+    const bf16_t* wa = gate_a + ((int64_t)b * block_size + 16 * ot + c) * block_size + 8 * g;
+    const bf16_t* wi = gate_i + ((int64_t)b * block_size + 16 * ot + c) * block_size + 8 * g;
+    f32x4 acc_a = f32x4{0.f, 0.f, 0.f, 0.f}, acc_i = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int kb = 0; kb < kbs; ++kb) {
+      const vf4 lo = *(const vf4*)(u_row + 32 * kb + 8 * g), hi = *(const vf4*)(u_row + 32 * kb + 8 * g + 4);
+      bf16x8 ub;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { ub[j] = (__bf16)lo[j]; ub[4 + j] = (__bf16)hi[j]; }
+      acc_a = MFMA16(*(const bf16x8*)(wa + 32 * kb), ub, acc_a);
+      acc_i = MFMA16(*(const bf16x8*)(wi + 32 * kb), ub, acc_i);
+    }
+    if (!live) continue;
+    const int o = 16 * ot + 4 * g, ch = b * block_size + o;      // the lane's four outputs of its row
+    vf4 va, vb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float r = 1.f / (1.f + expf(-(acc_a[i] + gate_a_bias[ch + i])));
+      const float gi = 1.f / (1.f + expf(-(acc_i[i] + gate_i_bias[ch + i])));
+      const float log_a = -decay_scale * soft_plus(lam[ch + i]) * r;
+      va[i] = expf(log_a);
+      vb[i] = sqrtf(-expm1f(2.f * log_a)) * gi * u_row[o + i];
+    }
+    float* dst = coef + row * 2 * width + ch;
+    *(vf4*)dst = va;
+    *(vf4*)(dst + width) = vb;
+  }
+}
+
 DRYFT_API int dryft_rglru_gates(const void* proj, int64_t proj_stride, int x_col, const float* x_bias,
                                 const float* conv_w, const float* conv_b, int taps, const void* gate_a,
                                 const float* gate_a_bias, const void* gate_i, const float* gate_i_bias,
@@ -259,6 +342,23 @@ DRYFT_API int dryft_rglru_gates(const void* proj, int64_t proj_stride, int x_col
   if (n_rows <= 0) return 0;
   if (blocks <= 0 || width % blocks || taps < 1 || taps > RG_MAX_TAPS) return -1;
   const int block_size = width / blocks;
+  // bfloat16 blocks of a multiple of 32 channels go to the matrix cores (16-byte pieces of the weights' rows)
+  const size_t mm_lds = (size_t)(n_rows <= 16 ? 16 : RG_MM_ROWS) * (block_size + RG_MM_PAD) * sizeof(float);
+  if (!is_f32 && block_size % 32 == 0 && mm_lds <= 150 * 1024 && width % 4 == 0 &&
+      (((uintptr_t)gate_a | (uintptr_t)gate_i | (uintptr_t)coef) & 15) == 0) {
+    const int few = n_rows <= 16;
+    const int tiles = block_size / 16;
+    dim3 mgrid(few ? 1 : (n_rows + RG_MM_ROWS - 1) / RG_MM_ROWS, blocks, few ? min(4, (tiles + 3) / 4) : 1);
+    if (mm_lds > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)rglru_gates_mfma_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)mm_lds) != hipSuccess)
+      return -1;
+    hipLaunchKernelGGL(rglru_gates_mfma_kernel, mgrid, dim3(256), mm_lds, stream, (const bf16_t*)proj, proj_stride,
+                       x_col, x_bias, conv_w, conv_b, taps, (const bf16_t*)gate_a, gate_a_bias, (const bf16_t*)gate_i,
+                       gate_i_bias, lam, decay_scale, row_slot, row_seq, row_pos, seq_start, tail, coef, n_rows, width,
+                       block_size, few);
+    return DRYFT_LAUNCH_CHECK();
+  }
   const size_t lds = (size_t)RG_ROWS * block_size * sizeof(float);
   if (lds > 64 * 1024) return -1;
   dim3 grid((n_rows + RG_ROWS - 1) / RG_ROWS, blocks), block(256);
