@@ -11,13 +11,16 @@
 // square, multiplies by a weight over all heads' features and by sigmoid(g), and rounds once.
 //
 // The recurrence kernel walks a sequence's rows of the step in order, whatever their number: a prompt, a
-// further portion of one, or one token. Grid (sequence, head, run of 63 value columns). A workgroup holds
-// its columns of S in registers, one column a lane, the rows of S dealt to its waves; lane 63 holds n as
-// one more column whose "value" is 1, so the same multiply-adds update it and the same reduction gives
-// n . q. Tokens are staged through LDS a tile at a time.
+// further portion of one, or one token. Grid (sequence, head, run of 64 value columns). A workgroup holds
+// its columns of S in registers, one column a lane, the rows of S dealt to its waves, and beside them n (every
+// lane of a wave the same entries), whose product with q goes through the same reduction as one more column.
+// Tokens are staged through LDS a tile at a time. n and m are kept once per run of 64 value columns
+// ([.., heads, runs, D] and [.., heads, runs]): every workgroup reads and writes its own copy, so none ever
+// reads what another has already updated.
 #include "common.h"
 
-#define MLSTM_COLS 63            // value columns a workgroup owns; lane 63 is the normaliser's
+#define MLSTM_COLS 64            // value columns a workgroup owns
+#define MLSTM_RED (MLSTM_COLS + 1)  // a wave's partial sums: its columns, then n . q
 #define MLSTM_TILE 16            // tokens staged at a time
 #define MLSTM_MAX_WAVES 16
 #define MLSTM_MAX_HELD 16        // rows of S a thread may hold: D <= waves * this
@@ -38,23 +41,25 @@ __global__ __launch_bounds__(1024) void mlstm_steps_kernel(
   const int waves = blockDim.x / WAVE, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int row0 = cu_rows[seq], n_tok = q_len[seq];
   const int col = c0 + lane;
-  const bool is_n = lane == MLSTM_COLS, is_v = !is_n && col < v_dim;
+  const bool is_v = col < v_dim;
+  const int runs = gridDim.z;
   float* qs = lds;                                        // [TILE][dim]
   float* ks = qs + MLSTM_TILE * dim;                      // [TILE][dim]
-  float* vs = ks + MLSTM_TILE * dim;                      // [TILE][64]: the workgroup's columns, 1 in the last
+  float* vs = ks + MLSTM_TILE * dim;                      // [TILE][64]: the workgroup's columns
   float* gi = vs + MLSTM_TILE * WAVE;                     // [TILE]
   float* gf = gi + MLSTM_TILE;                            // [TILE]
-  float* red = gf + MLSTM_TILE;                           // [2][waves][64]
+  float* red = gf + MLSTM_TILE;                           // [2][waves][65]
   const int64_t sh = (int64_t)slot * n_heads + head;
   float* S = state_s + sh * dim * v_dim;
-  float* N = state_n + sh * dim;
-  float held[HELD];
+  float* N = state_n + (sh * runs + blockIdx.z) * dim;
+  float held[HELD], held_n[HELD];
 #pragma unroll
   for (int j = 0; j < HELD; ++j) {
     const int d = wave + j * waves;
-    held[j] = d < dim ? (is_n ? N[d] : (is_v ? S[(int64_t)d * v_dim + col] : 0.f)) : 0.f;
+    held[j] = (d < dim && is_v) ? S[(int64_t)d * v_dim + col] : 0.f;
+    held_n[j] = d < dim ? N[d] : 0.f;
   }
-  float m = state_m[sh];
+  float m = state_m[sh * runs + blockIdx.z];
   for (int t0 = 0; t0 < n_tok; t0 += MLSTM_TILE) {
     const int nt = min(MLSTM_TILE, n_tok - t0);
     __syncthreads();                                      // the tile before is no longer read
@@ -67,8 +72,7 @@ __global__ __launch_bounds__(1024) void mlstm_steps_kernel(
     for (int e = threadIdx.x; e < nt * WAVE; e += blockDim.x) {
       const int t = e / WAVE, l = e % WAVE, c = c0 + l;
       float v = 0.f;
-      if (l == MLSTM_COLS) v = 1.f;
-      else if (c < v_dim) v = load_as_float(proj + (int64_t)(row0 + t0 + t) * proj_stride + v_col + (int64_t)head * v_dim + c);
+      if (c < v_dim) v = load_as_float(proj + (int64_t)(row0 + t0 + t) * proj_stride + v_col + (int64_t)head * v_dim + c);
       vs[e] = v;
     }
     if (threadIdx.x < nt) {
@@ -82,22 +86,27 @@ __global__ __launch_bounds__(1024) void mlstm_steps_kernel(
       const float keep = expf(gf[t] + m - m_new), take = expf(gi[t] - m_new);
       m = m_new;
       const float tv = take * vs[t * WAVE + lane];
-      float part = 0.f;
+      float part = 0.f, part_n = 0.f;
 #pragma unroll
       for (int j = 0; j < HELD; ++j) {
         const int d = wave + j * waves;
         if (d < dim) {
           held[j] = keep * held[j] + ks[t * dim + d] * tv;
+          held_n[j] = keep * held_n[j] + ks[t * dim + d] * take;
           part += held[j] * qs[t * dim + d];
+          part_n += held_n[j] * qs[t * dim + d];
         }
       }
-      float* r = red + ((t0 + t) & 1) * waves * WAVE;
-      r[wave * WAVE + lane] = part;
+      float* r = red + ((t0 + t) & 1) * waves * MLSTM_RED;
+      r[wave * MLSTM_RED + lane] = part;
+      if (lane == 0) r[wave * MLSTM_RED + MLSTM_COLS] = part_n;
       __syncthreads();                                    // one barrier a token: the two halves of `red` take turns
       if (wave == 0) {
-        float tot = 0.f;
-        for (int w = 0; w < waves; ++w) tot += r[w * WAVE + lane];
-        const float nq = __shfl(tot, MLSTM_COLS, WAVE);
+        float tot = 0.f, nq = 0.f;
+        for (int w = 0; w < waves; ++w) {
+          tot += r[w * MLSTM_RED + lane];
+          nq += r[w * MLSTM_RED + MLSTM_COLS];
+        }
         const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
         if (is_v) o_raw[((int64_t)(row0 + t0 + t) * n_heads + head) * v_dim + col] = tot / den;
       }
@@ -108,15 +117,15 @@ __global__ __launch_bounds__(1024) void mlstm_steps_kernel(
   for (int j = 0; j < HELD; ++j) {
     const int d = wave + j * waves;
     if (d < dim) {
-      if (is_n) { if (blockIdx.z == 0) N[d] = held[j]; }
-      else if (is_v) S[(int64_t)d * v_dim + col] = held[j];
+      if (is_v) S[(int64_t)d * v_dim + col] = held[j];
+      if (lane == 0) N[d] = held_n[j];
     }
   }
-  if (blockIdx.z == 0 && threadIdx.x == 0) state_m[sh] = m;
+  if (threadIdx.x == 0) state_m[sh * runs + blockIdx.z] = m;
 }
 
 DRYFT_API int dryft_mlstm_lds_bytes(int dim, int waves) {
-  return (2 * MLSTM_TILE * dim + MLSTM_TILE * WAVE + 2 * MLSTM_TILE + 2 * waves * WAVE) * (int)sizeof(float);
+  return (2 * MLSTM_TILE * dim + MLSTM_TILE * WAVE + 2 * MLSTM_TILE + 2 * waves * MLSTM_RED) * (int)sizeof(float);
 }
 
 // gates: float32 [rows, 2 * heads], the input gates' projections then the forget gates'. o_raw: float32
@@ -216,22 +225,54 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define CH_PAD 8
 #define CH_MAX_DT 4             // tiles of 16 key features a wave may own: D <= 256
 
-template <int KB>               // KB = ceil(D / 32)
+// Long prompts are also cut into segments of several chunks that run side by side, in two launches of this
+// kernel. MODE 1 walks every segment but a sequence's last from an empty memory (the first from the state the
+// step found, of which it also leaves a copy) and leaves what the segment makes of it: (S, n, m) and the sum B of
+// its log forget gates. Applying such a summary to a state (S_0, n_0, m_0) is m' = max(m_0 + B, m),
+// S' = exp(m_0 + B - m') S_0 + exp(m - m') S. MODE 2 folds the summaries before its segment into the state that
+// enters it, then walks its chunks as MODE 0 (one workgroup a sequence, no segments) does; a sequence's last
+// segment leaves the state. `tile_cu`: prefix sums over the sequences of their segments.
+struct Segments {
+  const int* tile_cu;
+  int n_seqs, seg_rows;
+  float *sum_s, *sum_n, *sum_m;       // [segments, heads, ...] as the state, and (m, B)
+  float *start_s, *start_n, *start_m; // [sequences, heads, ...]: the state the step found
+};
+
+template <int KB, int MODE>     // KB = ceil(D / 32)
 __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
     const bf16_t* __restrict__ proj, int64_t proj_stride, int q_col, int k_col, int v_col,
     const float* __restrict__ gates, const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
     const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
     float* __restrict__ state_s, float* __restrict__ state_n, float* __restrict__ state_m,
-    float* __restrict__ o_raw, int n_heads, int dim, int v_dim, float q_scale, int write_state) {
+    float* __restrict__ o_raw, int n_heads, int dim, int v_dim, float q_scale, int write_state, Segments sg) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int DP = 32 * KB;                                   // key features, padded with zeros
   constexpr int KS = DP + CH_PAD, TS = CH_L + CH_PAD;           // row strides in LDS
   constexpr int DT = (DP / 16 + 3) / 4;                         // key-feature tiles a wave owns
-  const int seq = blockIdx.x, head = blockIdx.y, v0 = blockIdx.z * CH_VS;
+  const int head = blockIdx.y, v0 = blockIdx.z * CH_VS;
+  int seq = blockIdx.x, seg = 0, seg_first = 0, n_segs = 1;
+  if (MODE != 0) {                                              // blockIdx.x counts segments over all sequences
+    if ((int)blockIdx.x >= sg.tile_cu[sg.n_seqs]) return;
+    int lo = 0, hi = sg.n_seqs;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (sg.tile_cu[mid] <= (int)blockIdx.x) lo = mid; else hi = mid;
+    }
+    while (lo + 1 < sg.n_seqs && sg.tile_cu[lo + 1] <= (int)blockIdx.x) ++lo;
+    seq = lo;
+    seg_first = sg.tile_cu[seq];
+    seg = blockIdx.x - seg_first;
+    n_segs = sg.tile_cu[seq + 1] - seg_first;
+  }
   const int slot = seq_slot[seq];
   if (slot < 0) return;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int row0 = cu_rows[seq], n_tok = q_len[seq];
+  const int tok_first = MODE == 0 ? 0 : seg * sg.seg_rows;
+  const int tok_end = MODE == 0 ? n_tok : min(n_tok, tok_first + sg.seg_rows);
+  const bool last_seg = seg == n_segs - 1;
+  if (MODE == 1 && last_seg && seg > 0) return;                 // nobody folds a sequence's last segment
   bf16_t* k_s = (bf16_t*)lds_raw;                               // [64][KS]      keys, row-wise
   bf16_t* kw_t = k_s + CH_L * KS;                               // [DP][TS]      (w_s k_s)^T, positions permuted
   bf16_t* v_t = kw_t + DP * TS;                                 // [64][TS]      V^T, positions permuted
@@ -243,7 +284,22 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   float* g_x = g_b + CH_L;                                      // [4]  M_L, b_L
   const int64_t sh = (int64_t)slot * n_heads + head;
   float* S = state_s + sh * dim * v_dim;
-  float* N = state_n + sh * dim;
+  float* N = state_n + (sh * gridDim.z + blockIdx.z) * dim;     // n and m: this run of value columns' own copy
+  float* M_state = state_m + sh * gridDim.z + blockIdx.z;
+  const int64_t per_s = (int64_t)dim * v_dim;
+  // where this workgroup's memory comes from: the state; in MODE 2 the copy MODE 1 left of it (a sequence of one
+  // segment reads the state itself: the workgroup that reads it is the one that writes it); nothing for a
+  // segment that MODE 1 walks from an empty memory; the first segment's summary for the later segments of MODE 2
+  const float* src_s = S;
+  const float* src_n = N;
+  const float* src_m = M_state;
+  if (MODE == 2 && n_segs > 1) {
+    const int64_t at = seg == 0 ? (int64_t)seq * n_heads + head : (int64_t)seg_first * n_heads + head;
+    src_s = (seg == 0 ? sg.start_s : sg.sum_s) + at * per_s;
+    src_n = (seg == 0 ? sg.start_n : sg.sum_n) + at * dim;
+    src_m = seg == 0 ? sg.start_m + at : sg.sum_m + 2 * at;
+  }
+  const bool empty = MODE == 1 && seg > 0;
   // the state: S^T tiles [value tile vt][own key-feature tile j], d-tile index = wave + 4 j
   f32x4 acc_s[4][DT];
 #pragma unroll
@@ -254,15 +310,59 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int v = v0 + 16 * vt + 4 * g + i;
-        acc_s[vt][j][i] = (d < dim && v < v_dim) ? S[(int64_t)d * v_dim + v] : 0.f;
+        acc_s[vt][j][i] = (!empty && d < dim && v < v_dim) ? src_s[(int64_t)d * v_dim + v] : 0.f;
       }
     }
-  for (int d = threadIdx.x; d < DP; d += blockDim.x) n_s[d] = d < dim ? N[d] : 0.f;
-  float m0 = state_m[sh];
-  for (int t0 = 0; t0 < n_tok; t0 += CH_L) {
-    const int nt = min(CH_L, n_tok - t0);
+  for (int d = threadIdx.x; d < DP; d += blockDim.x) n_s[d] = (!empty && d < dim) ? src_n[d] : 0.f;
+  float m0 = empty ? -INFINITY : src_m[0];
+  float b_sum = 0.f;
+  if (MODE == 1 && seg == 0) {                                  // the copy of the state the step found
+    const int64_t at = (int64_t)seq * n_heads + head;
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+      for (int j = 0; j < DT; ++j) {
+        const int d = 16 * (wave + 4 * j) + c;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int v = v0 + 16 * vt + 4 * g + i;
+          if (d < dim && v < v_dim) sg.start_s[at * per_s + (int64_t)d * v_dim + v] = acc_s[vt][j][i];
+        }
+      }
+    if (blockIdx.z == 0) {
+      for (int d = threadIdx.x; d < dim; d += blockDim.x) sg.start_n[at * dim + d] = src_n[d];
+      if (threadIdx.x == 0) sg.start_m[at] = m0;
+    }
+    if (last_seg) return;                                       // a sequence of one segment: MODE 2 does the rest
+  }
+  if (MODE == 2) {                                              // what the segments in between make of it
+    for (int k = 1; k < seg; ++k) {
+      const int64_t at = (int64_t)(seg_first + k) * n_heads + head;
+      const float mk = sg.sum_m[2 * at], bk = sg.sum_m[2 * at + 1];
+      const float m_new = fmaxf(m0 + bk, mk);
+      const float keep = expf(m0 + bk - m_new), take = expf(mk - m_new);
+      const float* ds = sg.sum_s + at * per_s;
+#pragma unroll
+      for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+        for (int j = 0; j < DT; ++j) {
+          const int d = 16 * (wave + 4 * j) + c;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int v = v0 + 16 * vt + 4 * g + i;
+            const float add = (d < dim && v < v_dim) ? ds[(int64_t)d * v_dim + v] : 0.f;
+            acc_s[vt][j][i] = keep * acc_s[vt][j][i] + take * add;
+          }
+        }
+      for (int d = threadIdx.x; d < dim; d += blockDim.x) n_s[d] = keep * n_s[d] + take * sg.sum_n[at * dim + d];
+      m0 = m_new;
+    }
+  }
+  for (int t0 = tok_first; t0 < tok_end; t0 += CH_L) {
+    const int nt = min(CH_L, tok_end - t0);
     __syncthreads();                                            // the chunk before is done with every buffer
     // S_0^T rounded, for the read-out of this chunk
+    if (MODE != 1)
 #pragma unroll
     for (int vt = 0; vt < 4; ++vt)
 #pragma unroll
@@ -319,6 +419,8 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
 #pragma unroll
       for (int j = 0; j < 8; ++j) v_t[(v + j) * TS + col] = float_to_bf16(vv[j]);
     }
+    if (MODE == 1) __syncthreads();                             // the chunk is staged
+    if (MODE != 1) {
     // this wave's 16 tokens: the queries stay in registers
     const int t = 16 * wave + c;                                // the lane's token of the chunk
     const bool t_live = t < nt;
@@ -396,6 +498,7 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
           }
       }
     }
+    }
     // the state after the chunk
     const float decay = expf(m0 - M_L);
 #pragma unroll
@@ -415,8 +518,29 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
       n_s[d] = a;
     }
     m0 = b_L + M_L;
+    b_sum += b_L;
   }
-  if (!write_state) return;
+  if (MODE == 1) {                                              // what the segment makes of a memory
+    const int64_t at = (int64_t)blockIdx.x * n_heads + head;
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt)
+#pragma unroll
+      for (int j = 0; j < DT; ++j) {
+        const int d = 16 * (wave + 4 * j) + c;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int v = v0 + 16 * vt + 4 * g + i;
+          if (d < dim && v < v_dim) sg.sum_s[at * per_s + (int64_t)d * v_dim + v] = acc_s[vt][j][i];
+        }
+      }
+    if (blockIdx.z == 0) {
+      __syncthreads();
+      for (int d = threadIdx.x; d < dim; d += blockDim.x) sg.sum_n[at * dim + d] = n_s[d];
+      if (threadIdx.x == 0) { sg.sum_m[2 * at] = m0; sg.sum_m[2 * at + 1] = b_sum; }
+    }
+    return;
+  }
+  if (!write_state || !last_seg) return;
 #pragma unroll
   for (int vt = 0; vt < 4; ++vt)
 #pragma unroll
@@ -429,11 +553,9 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
         if (v < v_dim) S[(int64_t)d * v_dim + v] = acc_s[vt][j][i];
       }
     }
-  if (blockIdx.z == 0) {
-    __syncthreads();
-    for (int d = threadIdx.x; d < dim; d += blockDim.x) N[d] = n_s[d];
-    if (threadIdx.x == 0) state_m[sh] = m0;
-  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < dim; d += blockDim.x) N[d] = n_s[d];
+  if (threadIdx.x == 0) M_state[0] = m0;
 }
 
 // Does the chunked kernel take these sizes? (16-byte pieces of rows; key width up to 256.)
@@ -442,28 +564,47 @@ DRYFT_API int dryft_mlstm_chunks_takes(int dim, int v_dim, int q_col, int k_col,
          v_col % 8 == 0 && proj_stride % 8 == 0;
 }
 
+// seg_rows == 0: one workgroup walks a whole sequence. Otherwise (a multiple of 64): sequences are cut into
+// segments of that many rows, `tile_cu` holding the prefix sums of their counts and `max_tiles` a bound on their
+// total, and `scratch` room for the summaries: (max_tiles + n_seqs) * heads * (dim * v_dim + dim + 2) floats.
 DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_col, int k_col, int v_col,
                                  const float* gates, const float* bias_i, const float* bias_f, float cap,
                                  const int* seq_slot, const int* cu_rows, const int* q_len, int n_seqs, float* state_s,
                                  float* state_n, float* state_m, float* o_raw, int n_heads, int dim, int v_dim,
-                                 float q_scale, int write_state, hipStream_t stream) {
+                                 float q_scale, int write_state, int seg_rows, const int* tile_cu, int max_tiles,
+                                 float* scratch, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (!dryft_mlstm_chunks_takes(dim, v_dim, q_col, k_col, v_col, proj_stride) || ((uintptr_t)proj & 15) || !(cap > 0.f))
+    return -1;
+  if (seg_rows < 0 || seg_rows % CH_L || (seg_rows > 0 && (tile_cu == nullptr || scratch == nullptr || max_tiles <= 0)))
     return -1;
   const int kb = (dim + 31) / 32, dp = 32 * kb;
   const size_t lds = (size_t)(2 * CH_L * (dp + CH_PAD) + dp * (CH_L + CH_PAD) + CH_VS * (CH_L + CH_PAD)) * 2 +
                      (size_t)(dp + 3 * CH_L + 4) * sizeof(float);
-  dim3 grid(n_seqs, n_heads, (v_dim + CH_VS - 1) / CH_VS), block(256);
-#define MC(KBV)                                                                                                      \
+  Segments sg = {};
+  if (seg_rows > 0) {
+    const size_t per = (size_t)n_heads * dim * v_dim, per_n = (size_t)n_heads * dim, per_m = (size_t)n_heads;
+    sg.tile_cu = tile_cu; sg.n_seqs = n_seqs; sg.seg_rows = seg_rows;
+    sg.sum_s = scratch;
+    sg.sum_n = sg.sum_s + max_tiles * per;
+    sg.sum_m = sg.sum_n + max_tiles * per_n;
+    sg.start_s = sg.sum_m + max_tiles * per_m * 2;
+    sg.start_n = sg.start_s + n_seqs * per;
+    sg.start_m = sg.start_n + n_seqs * per_n;
+  }
+  const int vs = (v_dim + CH_VS - 1) / CH_VS;
+#define MC1(KBV, MODEV, GRIDX)                                                                                        \
   {                                                                                                                  \
-    auto kernel = mlstm_chunks_kernel<KBV>;                                                                          \
+    auto kernel = mlstm_chunks_kernel<KBV, MODEV>;                                                                   \
     if (lds > 64 * 1024 &&                                                                                           \
         hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
       return -1;                                                                                                     \
-    hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)proj, proj_stride, q_col, k_col, v_col, gates, \
-                       bias_i, bias_f, cap, seq_slot, cu_rows, q_len, state_s, state_n, state_m, o_raw, n_heads, dim,  \
-                       v_dim, q_scale, write_state);                                                                 \
+    hipLaunchKernelGGL(kernel, dim3(GRIDX, n_heads, vs), dim3(256), lds, stream, (const bf16_t*)proj, proj_stride,   \
+                       q_col, k_col, v_col, gates, bias_i, bias_f, cap, seq_slot, cu_rows, q_len, state_s, state_n,    \
+                       state_m, o_raw, n_heads, dim, v_dim, q_scale, write_state, sg);                               \
   }
+#define MC(KBV)                                                                                                      \
+  if (seg_rows == 0) MC1(KBV, 0, n_seqs) else { MC1(KBV, 1, max_tiles) MC1(KBV, 2, max_tiles) }
   switch (kb) {
     case 1: MC(1); break;
     case 2: MC(2); break;
@@ -476,5 +617,6 @@ DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_co
     default: return -1;
   }
 #undef MC
+#undef MC1
   return DRYFT_LAUNCH_CHECK();
 }

@@ -31,7 +31,7 @@ _SIGNATURES = {
                                     _I, _I, _P],
               "dryft_mlstm_chunks_takes": [_I, _I, _I, _I, _I, _L],
               "dryft_mlstm_chunks": [_P, _L, _I, _I, _I, _P, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F,
-                                     _I, _P],
+                                     _I, _I, _P, _I, _P, _P],
               "dryft_mlstm_out": [_P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "rglru": {"dryft_rglru_gates": [_P, _L, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _F, _P, _P, _P, _P, _P, _P, _I, _I,
                                     _I, _I, _P],
@@ -1072,6 +1072,8 @@ def _seq_facts(seq_slot, cu_rows, q_len, n_seqs: int) -> None:
 
 
 MLSTM_MAX_DIM = 256
+MLSTM_COLUMNS = 64       # value columns a workgroup of either kernel owns
+MLSTM_CHUNK = 64         # tokens the chunked kernel takes at a time; segments are multiples of it
 
 
 def mlstm_chunks_takes(proj, q_col: int, k_col: int, v_col: int, dim: int, v_dim: int) -> bool:
@@ -1082,11 +1084,12 @@ def mlstm_chunks_takes(proj, q_col: int, k_col: int, v_col: int, dim: int, v_dim
 
 def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f, cap: float, seq_slot, cu_rows, q_len,
                 n_seqs: int, state_s, state_n, state_m, o_raw, n_heads: int, dim: int, v_dim: int, q_scale: float,
-                write_state: bool, chunked: bool = False) -> None:
+                write_state: bool, chunked: bool = False, segments: tuple | None = None) -> None:
     """The matrix-memory recurrence over each sequence's rows of the step, in order; ``o_raw`` (float32
     ``[rows, heads, v_dim]``) receives each token's read-out divided by its normaliser. ``gates`` are the float32
     projections ``[rows, 2 * heads]`` (input gates, then forget gates) before bias, cap and log-sigmoid. The states
-    ``[slots, heads, dim, v_dim]``, ``[slots, heads, dim]`` and ``[slots, heads]`` are float32."""
+    ``[slots, heads, dim, v_dim]``, ``[slots, heads, runs, dim]`` and ``[slots, heads, runs]`` are float32, the
+    normaliser and the maximum once per run of ``MLSTM_COLUMNS`` value columns (each workgroup keeps its own)."""
     _gpu(proj, "proj")
     is_f32 = _float_flag(proj, "proj")
     rows = proj.shape[0]
@@ -1104,8 +1107,9 @@ def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f,
     _f32_vector(bias_f, "bias_f", n_heads)
     _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
     slots = state_m.shape[0]
-    for name, t, shape in (("state_s", state_s, (slots, n_heads, dim, v_dim)), ("state_n", state_n, (slots, n_heads, dim)),
-                           ("state_m", state_m, (slots, n_heads))):
+    runs = -(-v_dim // MLSTM_COLUMNS)
+    for name, t, shape in (("state_s", state_s, (slots, n_heads, dim, v_dim)),
+                           ("state_n", state_n, (slots, n_heads, runs, dim)), ("state_m", state_m, (slots, n_heads, runs))):
         _gpu(t, name, torch.float32)
         if not (tuple(t.shape) == shape and t.is_contiguous()):
             raise KernelError(f"{name}: must be contiguous float32 {shape}, got {tuple(t.shape)}")
@@ -1116,10 +1120,23 @@ def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f,
         # the same recurrence a chunk of 64 tokens at a time on the matrix cores (steps of many rows, bfloat16)
         if not mlstm_chunks_takes(proj, q_col, k_col, v_col, dim, v_dim):
             raise KernelError("mlstm_steps: the chunked kernel does not take these sizes")
+        # ``segments`` = (rows a segment, tile_cu, bound on the segments): long sequences cut into segments that run
+        # side by side, in two launches with summaries of the segments in between
+        seg_rows, tile_cu, max_tiles, scratch = 0, None, 0, None
+        if segments is not None:
+            seg_rows, tile_cu, max_tiles = segments
+            if seg_rows <= 0 or seg_rows % MLSTM_CHUNK or max_tiles <= 0:
+                raise KernelError(f"mlstm_steps: segments of {seg_rows} rows, at most {max_tiles} of them")
+            _gpu(tile_cu, "tile_cu", torch.int32)
+            if not (tile_cu.is_contiguous() and tile_cu.numel() >= n_seqs + 1):
+                raise KernelError(f"tile_cu: needs {n_seqs + 1} contiguous entries")
+            scratch = torch.empty((max_tiles + n_seqs) * n_heads * (dim * v_dim + dim + 2), dtype=torch.float32,
+                                  device=proj.device)
         _check(_fn("mlstm", "dryft_mlstm_chunks")(
             _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),
             _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs, _ptr(state_s), _ptr(state_n), _ptr(state_m),
-            _ptr(o_raw), n_heads, dim, v_dim, float(q_scale), int(bool(write_state)), _stream()), "mlstm_chunks")
+            _ptr(o_raw), n_heads, dim, v_dim, float(q_scale), int(bool(write_state)), seg_rows, _ptr(tile_cu),
+            max_tiles, _ptr(scratch), _stream()), "mlstm_chunks")
         return
     _check(_fn("mlstm", "dryft_mlstm_steps")(
         _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),

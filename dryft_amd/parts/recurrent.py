@@ -25,6 +25,7 @@ from .base import Mixer, StepContext, matrix
 from .linear import linear
 
 
+_MAX_SEGMENTS = 8
 _CHUNKED_FROM = 8       # steps whose longest sequence brings more rows than this take the chunked matrix-memory kernel
 
 
@@ -63,8 +64,11 @@ class MatrixMemory(Mixer):
         self.out_norm = tensors["out_norm"].float().contiguous()
 
     def cache_need(self):
+        # the normaliser and the maximum once per run of value columns that a workgroup owns, so that no workgroup
+        # reads what another has already updated
+        runs = -(-self.value_dim // ops.MLSTM_COLUMNS)
         return {"memory": StateNeed((self.n_heads, self.key_dim, self.value_dim)),
-                "normaliser": StateNeed((self.n_heads, self.key_dim)), "maximum": StateNeed((self.n_heads,))}
+                "normaliser": StateNeed((self.n_heads, runs, self.key_dim)), "maximum": StateNeed((self.n_heads, runs))}
 
     def kernel_modules(self, dtype):
         return ("gemm", "mlstm")
@@ -81,11 +85,24 @@ class MatrixMemory(Mixer):
         ops.mlstm_steps(proj, 0, self.qk_dim, 2 * self.qk_dim, gates, self.bias_i, self.bias_f, self.gate_cap,
                         ctx.seq_slot, ctx.cu_rows, ctx.q_len, ctx.n_seqs, line["memory"].state,
                         line["normaliser"].state, line["maximum"].state, o_raw, self.n_heads, self.key_dim,
-                        self.value_dim, self.key_dim ** -0.5, writes_cache, chunked=chunked)
+                        self.value_dim, self.key_dim ** -0.5, writes_cache, chunked=chunked,
+                        segments=self._segments(ctx) if chunked else None)
         out = torch.empty((rows, self.v_dim), dtype=h.dtype, device=h.device)
         ops.mlstm_out(o_raw, proj, 2 * self.qk_dim + self.v_dim, self.out_norm, ctx.row_slot, out, self.n_heads,
                       self.value_dim, self.norm_eps)
         return linear(out, self.w_o, allow_partials=True)
+
+    @staticmethod
+    def _segments(ctx: StepContext):
+        """How the chunked kernel cuts long sequences: into at most ``_MAX_SEGMENTS`` segments of whole chunks each
+        (a later segment folds the summaries of all before it, so few are better than many), none for sequences
+        of at most two chunks."""
+        chunks = -(-ctx.max_q_len // ops.MLSTM_CHUNK)
+        if chunks <= 2:
+            return None
+        seg_rows = ops.MLSTM_CHUNK * max(2, -(-chunks // _MAX_SEGMENTS))
+        tile_cu, max_tiles = ctx.tiles(seg_rows)
+        return seg_rows, tile_cu, max_tiles
 
     def flops(self, rows, spans):
         """The projections, and per token and head the update of the memory and its read-out."""
