@@ -281,7 +281,8 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   float* g_M = n_s + DP;                                        // [64] M_t
   float* g_c = g_M + CH_L;                                      // [64] c_s
   float* g_b = g_c + CH_L;                                      // [64] b_t
-  float* g_x = g_b + CH_L;                                      // [4]  M_L, b_L
+  float* g_w = g_b + CH_L;                                      // [64] w_s = exp(c_s - M_L)
+  float* g_x = g_w + CH_L;                                      // [4]  M_L, b_L
   const int64_t sh = (int64_t)slot * n_heads + head;
   float* S = state_s + sh * dim * v_dim;
   float* N = state_n + (sh * gridDim.z + blockIdx.z) * dim;     // n and m: this run of value columns' own copy
@@ -394,24 +395,27 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
       g_M[lane] = M;
       g_c[lane] = cs;
       g_b[lane] = b;
+      g_w[lane] = live ? expf(cs - __shfl(M, nt - 1, WAVE)) : 0.f;
       if (lane == nt - 1) { g_x[0] = M; g_x[1] = b; }
     }
     __syncthreads();
     const float M_L = g_x[0], b_L = g_x[1];
     // stage the chunk: K row-wise; (w_s k_s)^T and V^T with the positions in the lanes' order
+    // (neighbouring threads take neighbouring positions of the same features: their 2-byte writes into the
+    // transposed copies then fall into one row, not into rows that share banks)
     for (int e = threadIdx.x; e < CH_L * (DP / 8); e += blockDim.x) {
-      const int s = e / (DP / 8), d = 8 * (e % (DP / 8));
+      const int s = e % CH_L, d = 8 * (e / CH_L);
       float kv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (s < nt && d < dim)                                    // dim is a multiple of 8 (the host checks)
         load8_as_float(proj + (int64_t)(row0 + t0 + s) * proj_stride + k_col + (int64_t)head * dim + d, kv);
       store8_from_float(k_s + s * KS + d, kv);
-      const float w = s < nt ? expf(g_c[s] - M_L) : 0.f;
+      const float w = g_w[s];
       const int col = value_column(s);
 #pragma unroll
       for (int j = 0; j < 8; ++j) kw_t[(d + j) * TS + col] = float_to_bf16(w * kv[j]);
     }
     for (int e = threadIdx.x; e < CH_L * (CH_VS / 8); e += blockDim.x) {
-      const int s = e / (CH_VS / 8), v = 8 * (e % (CH_VS / 8));
+      const int s = e % CH_L, v = 8 * (e / CH_L);
       float vv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (s < nt && v0 + v < v_dim)                             // v_dim is a multiple of 8
         load8_as_float(proj + (int64_t)(row0 + t0 + s) * proj_stride + v_col + (int64_t)head * v_dim + v0 + v, vv);
@@ -514,7 +518,7 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
       }
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {
       float a = decay * n_s[d];
-      for (int s = 0; s < nt; ++s) a += expf(g_c[s] - M_L) * bf16_to_float(k_s[s * KS + d]);
+      for (int s = 0; s < nt; ++s) a += g_w[s] * bf16_to_float(k_s[s * KS + d]);
       n_s[d] = a;
     }
     m0 = b_L + M_L;
@@ -580,7 +584,7 @@ DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_co
     return -1;
   const int kb = (dim + 31) / 32, dp = 32 * kb;
   const size_t lds = (size_t)(2 * CH_L * (dp + CH_PAD) + dp * (CH_L + CH_PAD) + CH_VS * (CH_L + CH_PAD)) * 2 +
-                     (size_t)(dp + 3 * CH_L + 4) * sizeof(float);
+                     (size_t)(dp + 4 * CH_L + 4) * sizeof(float);
   Segments sg = {};
   if (seg_rows > 0) {
     const size_t per = (size_t)n_heads * dim * v_dim, per_n = (size_t)n_heads * dim, per_m = (size_t)n_heads;

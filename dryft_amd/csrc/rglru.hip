@@ -275,25 +275,60 @@ __global__ __launch_bounds__(256) void rglru_gates_mfma_kernel(
   const int wg_rows = few ? 16 : RG_MM_ROWS;
   const int r0 = blockIdx.x * wg_rows, b = blockIdx.y, ld = block_size + RG_MM_PAD;
   const int rows = min(wg_rows, n_rows - r0);
-  for (int e = threadIdx.x; e < wg_rows * block_size; e += blockDim.x) {
-    const int rr = e / block_size, cc = e % block_size, ch = b * block_size + cc;
-    float u = 0.f;
-    if (rr < rows) {
-      const int64_t row = r0 + rr;
-      const int slot = row_slot[row];
-      if (slot >= 0) {
-        const int pos = row_pos[row], start = seq_start[row_seq[row]];
-        u = conv_b[ch];
-        for (int j = 0; j < taps; ++j) {
-          const int back = taps - 1 - j, p = pos - back;
-          float x;
-          if (p >= start) x = load_as_float(proj + (row - back) * proj_stride + x_col + ch) + x_bias[ch];
-          else x = tail[((int64_t)slot * (taps - 1) + (taps - 1 - start + p)) * width + ch];
-          u += conv_w[ch * taps + j] * x;
+  // the rows' facts once; then a thread takes one channel and walks a run of the rows in order, so that the
+  // convolution's window slides: a row that follows its predecessor in the same sequence brings one new input
+  __shared__ int r_slot[RG_MM_ROWS], r_pos[RG_MM_ROWS], r_start[RG_MM_ROWS];
+  if (threadIdx.x < wg_rows) {
+    int slot = -1, pos = 0, start = 0;
+    if ((int)threadIdx.x < rows) {
+      const int64_t row = r0 + threadIdx.x;
+      slot = row_slot[row];
+      if (slot >= 0) { pos = row_pos[row]; start = seq_start[row_seq[row]]; }
+    }
+    r_slot[threadIdx.x] = slot; r_pos[threadIdx.x] = pos; r_start[threadIdx.x] = start;
+  }
+  __syncthreads();
+  {
+    const int ch_threads = min(block_size, (int)blockDim.x), groups = blockDim.x / ch_threads;
+    const int grp = threadIdx.x / ch_threads, per = (wg_rows + groups - 1) / groups;
+    const int rr0 = grp * per, rr1 = grp < groups ? min(wg_rows, rr0 + per) : 0;
+    for (int cc = threadIdx.x % ch_threads; cc < block_size && rr0 < rr1; cc += ch_threads) {
+      const int ch = b * block_size + cc;
+      // taps and window sit at the end of arrays of fixed size (place k holds the input `15 - k` positions back)
+      float cw[RG_MAX_TAPS], win[RG_MAX_TAPS];
+#pragma unroll
+      for (int k = 0; k < RG_MAX_TAPS; ++k) {
+        cw[k] = k >= RG_MAX_TAPS - taps ? conv_w[ch * taps + k - (RG_MAX_TAPS - taps)] : 0.f;
+        win[k] = 0.f;
+      }
+      const float xb = x_bias[ch], cb = conv_b[ch];
+      for (int rr = rr0; rr < rr1; ++rr) {
+        const int slot = r_slot[rr];
+        float u = 0.f;
+        if (slot >= 0) {
+          const int pos = r_pos[rr], start = r_start[rr];
+          const int64_t row = r0 + rr;
+          const bool slides = rr > rr0 && r_slot[rr - 1] == slot && r_pos[rr - 1] == pos - 1;
+          if (slides) {
+#pragma unroll
+            for (int k = 0; k < RG_MAX_TAPS - 1; ++k) win[k] = win[k + 1];
+            win[RG_MAX_TAPS - 1] = load_as_float(proj + row * proj_stride + x_col + ch) + xb;
+          } else {
+#pragma unroll
+            for (int k = 0; k < RG_MAX_TAPS; ++k) {
+              if (k < RG_MAX_TAPS - taps) continue;
+              const int back = RG_MAX_TAPS - 1 - k, p = pos - back;
+              if (p >= start) win[k] = load_as_float(proj + (row - back) * proj_stride + x_col + ch) + xb;
+              else win[k] = tail[((int64_t)slot * (taps - 1) + (taps - 1 - start + p)) * width + ch];  // zeros before the start
+            }
+          }
+          u = cb;
+#pragma unroll
+          for (int k = 0; k < RG_MAX_TAPS; ++k) u += cw[k] * win[k];
         }
+        u_s[rr * ld + cc] = u;
       }
     }
-    u_s[rr * ld + cc] = u;
   }
   __syncthreads();
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
