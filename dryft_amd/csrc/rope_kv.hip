@@ -512,11 +512,11 @@ __global__ __launch_bounds__(256) void rope_pairs_kv_kernel(const T* __restrict_
                                                             T* __restrict__ k_pages, T* __restrict__ v_pages,
                                                             const int* __restrict__ page_table, int max_pages,
                                                             int write_kv, int n_heads, int n_kv, int head_dim,
-                                                            int v_dim) {
+                                                            int v_dim, int skip_v) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = blockIdx.x;
   const int job = blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
-  if (job >= n_heads + 2 * n_kv) return;
+  if (job >= n_heads + (skip_v ? 1 : 2) * n_kv) return;   // skip_v: the values go through the tile kernel
   const int slot = row_slot[row], pos = row_pos[row];
   const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
   if (is_q) {
@@ -562,14 +562,27 @@ DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_c
                                   int n_kv, int head_dim, int v_dim, int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (rot < 0 || rot % 2 || rot > head_dim || n_kv <= 0 || q_out == nullptr) return -1;
-  dim3 grid(n_rows, (n_heads + 2 * n_kv + 3) / 4), block(256);
+  // many rows: the values are transposed a tile of 64 rows at a time instead of 2 bytes at a time
+  const size_t v_lds = (size_t)v_dim * V_TILE_LD * (is_f32 ? 4 : 2);
+  const int skip_v = (write_kv && n_rows >= 32 && v_dim % 8 == 0 && v_col % 8 == 0 && proj_stride % 8 == 0 &&
+                      (((uintptr_t)proj | (uintptr_t)v_pages) & 15) == 0 && v_lds <= 64 * 1024) ? 1 : 0;
+  dim3 grid(n_rows, (n_heads + (skip_v ? 1 : 2) * n_kv + 3) / 4), block(256);
   if (is_f32)
     hipLaunchKernelGGL(rope_pairs_kv_kernel<float>, grid, block, 0, stream, (const float*)proj, proj_stride, q_col,
                        k_col, v_col, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages,
-                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim);
+                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v);
   else
     hipLaunchKernelGGL(rope_pairs_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)proj, proj_stride, q_col,
                        k_col, v_col, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out, (bf16_t*)k_pages,
-                       (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim);
+                       (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v);
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc || !skip_v) return rc;
+  dim3 vgrid((n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS, n_kv);
+  if (is_f32)
+    hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, dim3(256), v_lds, stream, (const float*)proj, proj_stride,
+                       v_col, row_slot, row_pos, (float*)v_pages, page_table, max_pages, n_rows, n_kv, v_dim);
+  else
+    hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, dim3(256), v_lds, stream, (const bf16_t*)proj, proj_stride,
+                       v_col, row_slot, row_pos, (bf16_t*)v_pages, page_table, max_pages, n_rows, n_kv, v_dim);
   return DRYFT_LAUNCH_CHECK();
 }
