@@ -163,7 +163,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void mlstm_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ proj,
                                                         int64_t proj_stride, int g_col, const float* __restrict__ w,
                                                         const int* __restrict__ row_slot, T* __restrict__ out,
-                                                        int n_heads, int v_dim, float eps) {
+                                                        int n_heads, int v_dim, float eps, int vec) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = blockIdx.x;
   const int head = blockIdx.y * 4 + wave;
@@ -174,10 +174,29 @@ __global__ __launch_bounds__(256) void mlstm_out_kernel(const float* __restrict_
     return;
   }
   const float* o = o_raw + (row * n_heads + head) * v_dim;
+  const T* g = proj + row * proj_stride + g_col + (int64_t)head * v_dim;
+  if (vec) {                                               // 8 values a lane, 16 bytes a load (widths of 8 up to 512)
+    const int c = 8 * lane;
+    float ov[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, gv[8], wv[8];
+    float ss = 0.f;
+    if (c < v_dim) {
+      load8_as_float(o + c, ov);
+      load8_as_float(g + c, gv);
+      load8_as_float(w + head * v_dim + c, wv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += ov[j] * ov[j];
+    }
+    const float inv = rsqrtf(wave_sum(ss) / (float)v_dim + eps);
+    if (c < v_dim) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ov[j] = ov[j] * inv * wv[j] / (1.f + expf(-gv[j]));
+      store8_from_float(dst + c, ov);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int c = lane; c < v_dim; c += WAVE) ss += o[c] * o[c];
   const float inv = rsqrtf(wave_sum(ss) / (float)v_dim + eps);
-  const T* g = proj + row * proj_stride + g_col + (int64_t)head * v_dim;
   for (int c = lane; c < v_dim; c += WAVE) {
     const float gate = 1.f / (1.f + expf(-load_as_float(g + c)));
     store_from_float(dst + c, o[c] * inv * w[head * v_dim + c] * gate);
@@ -189,12 +208,14 @@ DRYFT_API int dryft_mlstm_out(const float* o_raw, const void* proj, int64_t proj
                               int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   dim3 grid(n_rows, (n_heads + 3) / 4), block(256);
+  const int vec = v_dim % 8 == 0 && v_dim <= 8 * WAVE && g_col % 8 == 0 && proj_stride % 8 == 0 &&
+                  (((uintptr_t)o_raw | (uintptr_t)proj | (uintptr_t)w | (uintptr_t)out) & 15) == 0;
   if (is_f32)
     hipLaunchKernelGGL(mlstm_out_kernel<float>, grid, block, 0, stream, o_raw, (const float*)proj, proj_stride, g_col,
-                       w, row_slot, (float*)out, n_heads, v_dim, eps);
+                       w, row_slot, (float*)out, n_heads, v_dim, eps, vec);
   else
     hipLaunchKernelGGL(mlstm_out_kernel<bf16_t>, grid, block, 0, stream, o_raw, (const bf16_t*)proj, proj_stride,
-                       g_col, w, row_slot, (bf16_t*)out, n_heads, v_dim, eps);
+                       g_col, w, row_slot, (bf16_t*)out, n_heads, v_dim, eps, vec);
   return DRYFT_LAUNCH_CHECK();
 }
 

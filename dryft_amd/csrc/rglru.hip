@@ -155,10 +155,19 @@ __global__ __launch_bounds__(256) void rglru_tile_ends_kernel(const float* __res
   if (!rg_locate(blockIdx.x, tile_cu, n_seqs, seq, j) || ch >= width) return;
   const int t0 = j * RG_TILE, t1 = min(q_len[seq], t0 + RG_TILE);
   float P = 1.f, Q = 0.f;
-  for (int t = t0; t < t1; ++t) {
-    const float* c = coef + (int64_t)(cu_rows[seq] + t) * 2 * width;
-    P *= c[ch];
-    Q = c[ch] * Q + c[width + ch];
+  const float* c0 = coef + (int64_t)cu_rows[seq] * 2 * width + ch;
+  int t = t0;
+  for (; t + 8 <= t1; t += 8) {                                 // eight tokens' coefficients asked for together
+    float a[8], bb[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { a[u] = c0[(int64_t)(t + u) * 2 * width]; bb[u] = c0[(int64_t)(t + u) * 2 * width + width]; }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { P *= a[u]; Q = a[u] * Q + bb[u]; }
+  }
+  for (; t < t1; ++t) {
+    const float a = c0[(int64_t)t * 2 * width], bb = c0[(int64_t)t * 2 * width + width];
+    P *= a;
+    Q = a * Q + bb;
   }
   ends[((int64_t)blockIdx.x * 2) * width + ch] = P;
   ends[((int64_t)blockIdx.x * 2 + 1) * width + ch] = Q;
@@ -209,8 +218,25 @@ __global__ __launch_bounds__(256) void rglru_apply_tiles_kernel(
   float S = ends[((int64_t)blockIdx.x * 2) * width + ch];
   const float yb = y_bias[ch];
   const int t0 = j * RG_TILE, t1 = min(q_len[seq], t0 + RG_TILE);
-  for (int t = t0; t < t1; ++t) {
-    const int64_t row = cu_rows[seq] + t;
+  const int64_t first = cu_rows[seq];
+  int t = t0;
+  for (; t + 8 <= t1; t += 8) {                                 // eight tokens' operands asked for together
+    float a[8], bb[8], y[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t row = first + t + u;
+      a[u] = coef[row * 2 * width + ch];
+      bb[u] = coef[row * 2 * width + width + ch];
+      y[u] = load_as_float(proj + row * proj_stride + y_col + ch);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      S = a[u] * S + bb[u];
+      store_from_float(out + (first + t + u) * width + ch, S * gelu_tanh(y[u] + yb));
+    }
+  }
+  for (; t < t1; ++t) {
+    const int64_t row = first + t;
     const float* c = coef + row * 2 * width;
     S = c[ch] * S + c[width + ch];
     const float y = gelu_tanh(load_as_float(proj + row * proj_stride + y_col + ch) + yb);
