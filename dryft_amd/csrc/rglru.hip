@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void rglru_apply_tiles_kernel(
   }
 }
 
-DRYFT_API int dryft_rglru_tile_rows(void) { return RG_TILE; }
+DRYFT_API int dryft_rglru_tile_rows() { return RG_TILE; }
 
 // out must hold zeros (or anything finite) in the rows of sequences that sit out: no tile visits them.
 DRYFT_API int dryft_rglru_scan_tiles(const float* coef, float* ends, const void* proj, int64_t proj_stride, int x_col,
