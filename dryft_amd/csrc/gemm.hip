@@ -574,16 +574,28 @@ __device__ __forceinline__ float silu_for_bf16(float g) {
 // n .. n + 3 (n = first + 4 g), the lane 32 further on their ups. The two lanes share the work: the first takes
 // outputs n and n + 1, the second n + 2 and n + 3, each after one exchange of two values.
 // y[n + i] = T(T(silu(gate)) * up), two values in one store where N is even.
+// With `act.limit` > 0 the unit is the clamped one instead: g = min(gate, limit), u = clamp(up, -limit, limit),
+// y = T(g * sigmoid(alpha g) * (u + 1)), from the float accumulators, rounded once.
+struct GateAct {
+  float limit = 0.f, alpha = 0.f;
+};
+__device__ __forceinline__ float clamped_unit(float gate, float up, const GateAct& act) {
+  const float gc = fminf(gate, act.limit), uc = fminf(fmaxf(up, -act.limit), act.limit);
+  return gc * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(gc * act.alpha * -1.4426950408889634f)) * (uc + 1.f);
+}
 __device__ __forceinline__ void swiglu_store4(bf16_t* __restrict__ y_row, int first, int N, int g, const f32x4& acc,
-                                              bool row_there) {
+                                              bool row_there, GateAct act = {}) {
   const bool second = g >= 2;
   const float got0 = __shfl_xor(second ? acc[0] : acc[2], 32, WAVE);
   const float got1 = __shfl_xor(second ? acc[1] : acc[3], 32, WAVE);
   const float gate0 = second ? got0 : acc[0], gate1 = second ? got1 : acc[1];
   const float up0 = second ? acc[2] : got0, up1 = second ? acc[3] : got1;
   const int n = first + 4 * (g & 1) + (second ? 2 : 0);
-  const bf16_t v0 = float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate0))) * rounded_as<bf16_t>(up0));
-  const bf16_t v1 = float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate1))) * rounded_as<bf16_t>(up1));
+  const bool clamped = act.limit > 0.f;
+  const bf16_t v0 = clamped ? float_to_bf16(clamped_unit(gate0, up0, act))
+                            : float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate0))) * rounded_as<bf16_t>(up0));
+  const bf16_t v1 = clamped ? float_to_bf16(clamped_unit(gate1, up1, act))
+                            : float_to_bf16(rounded_as<bf16_t>(silu_for_bf16(rounded_as<bf16_t>(gate1))) * rounded_as<bf16_t>(up1));
   if (!row_there || n >= N) return;
   if (N % 2 == 0) {                                        // then n + 1 < N too, and the address is a multiple of 4
     *(uint32_t*)(y_row + n) = (uint32_t)v0.bits | ((uint32_t)v1.bits << 16);
@@ -602,7 +614,8 @@ __device__ __forceinline__ void swiglu_store4(bf16_t* __restrict__ y_row, int fi
 template <int MT, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gemm_panel_swiglu_kernel(const bf16_t* __restrict__ x, int64_t x_stride,
                                                                        const bf16_t* __restrict__ w,
-                                                                       bf16_t* __restrict__ y, int M, int N, int K) {
+                                                                       bf16_t* __restrict__ y, int M, int N, int K,
+                                                                       GateAct act) {
   extern __shared__ __align__(16) unsigned char panel_lds[];
   constexpr int STAGES = PANEL_STAGES;
   constexpr int RB = 2 * PANEL_GROUP;                      // bytes of a row in a group
@@ -697,13 +710,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_panel_swiglu_kernel(const bf1
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + c;
-    swiglu_store4(y + (int64_t)min(m, M - 1) * N, n0, N, g, acc[mt], m < M);
+    swiglu_store4(y + (int64_t)min(m, M - 1) * N, n0, N, g, acc[mt], m < M, act);
   }
 }
 
 template <int MT, int WAVES>
 static int launch_panel_swiglu(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
-                               hipStream_t stream) {
+                               hipStream_t stream, GateAct act) {
   constexpr int lds = PANEL_STAGES * (16 * WAVES + 16 * MT) * 2 * PANEL_GROUP;
   static_assert(lds <= 160 * 1024, "the stages must fit a compute unit's LDS");
   static bool raised = false;                              // more dynamic LDS than the default limit allows
@@ -713,19 +726,20 @@ static int launch_panel_swiglu(const void* x, int64_t x_stride, const void* w, v
     raised = true;
   }
   dim3 grid((N + 8 * WAVES - 1) / (8 * WAVES)), block(64 * WAVES);
-  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (bf16_t*)y, M, N, K);
+  hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)x, x_stride, (const bf16_t*)w, (bf16_t*)y, M, N, K,
+                     act);
   return DRYFT_LAUNCH_CHECK();
 }
 
 template <int MT>
 static int panel_waves(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int waves,
-                       hipStream_t stream) {
+                       hipStream_t stream, GateAct act) {
   switch (waves) {
-    case 4: return launch_panel_swiglu<MT, 4>(x, x_stride, w, y, M, N, K, stream);
-    case 5: return launch_panel_swiglu<MT, 5>(x, x_stride, w, y, M, N, K, stream);
-    case 6: return launch_panel_swiglu<MT, 6>(x, x_stride, w, y, M, N, K, stream);
-    case 7: return launch_panel_swiglu<MT, 7>(x, x_stride, w, y, M, N, K, stream);
-    case 8: return launch_panel_swiglu<MT, 8>(x, x_stride, w, y, M, N, K, stream);
+    case 4: return launch_panel_swiglu<MT, 4>(x, x_stride, w, y, M, N, K, stream, act);
+    case 5: return launch_panel_swiglu<MT, 5>(x, x_stride, w, y, M, N, K, stream, act);
+    case 6: return launch_panel_swiglu<MT, 6>(x, x_stride, w, y, M, N, K, stream, act);
+    case 7: return launch_panel_swiglu<MT, 7>(x, x_stride, w, y, M, N, K, stream, act);
+    case 8: return launch_panel_swiglu<MT, 8>(x, x_stride, w, y, M, N, K, stream, act);
     default: return -1;
   }
 }
@@ -750,18 +764,37 @@ DRYFT_API int dryft_gemm_panel_waves(int N) {
 
 // M <= 64. y[M, N] = T(T(silu(x . Wg^T)) * (x . Wu^T)) with W = [Wg; Wu] of 2N rows; K a multiple of 128; x and W
 // within reach of 32-bit byte offsets; waves: 4 to 8, or 0 for dryft_gemm_panel_waves' choice.
+static int panel_entry(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int waves,
+                       GateAct act, hipStream_t stream);
+
 DRYFT_API int dryft_gemm_panel_swiglu_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K,
                                            int waves, hipStream_t stream) {
+  return panel_entry(x, x_stride, w, y, M, N, K, waves, GateAct{}, stream);
+}
+
+// The same product with the clamped gated unit in its epilogue: y = T(g sigmoid(alpha g) (u + 1)),
+// g = min(x . Wg^T, limit), u = clamp(x . Wu^T, -limit, limit); limit > 0.
+DRYFT_API int dryft_gemm_panel_glu_clamped_bf16(const void* x, int64_t x_stride, const void* w, void* y, int M, int N,
+                                                int K, int waves, float limit, float alpha, hipStream_t stream) {
+  if (!(limit > 0.f)) return -1;
+  GateAct act;
+  act.limit = limit;
+  act.alpha = alpha;
+  return panel_entry(x, x_stride, w, y, M, N, K, waves, act, stream);
+}
+
+static int panel_entry(const void* x, int64_t x_stride, const void* w, void* y, int M, int N, int K, int waves,
+                       GateAct act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % PANEL_GROUP || x_stride % 8 || (((uintptr_t)x | (uintptr_t)w) & 15) ||
       (int64_t)2 * N * K * 2 >= (int64_t)4 << 30 || (int64_t)M * x_stride * 2 >= (int64_t)4 << 30)
     return -1;
   if (waves == 0) waves = dryft_gemm_panel_waves(N);
   switch ((M + 15) / 16) {
-    case 1: return panel_waves<1>(x, x_stride, w, y, M, N, K, waves, stream);
-    case 2: return panel_waves<2>(x, x_stride, w, y, M, N, K, waves, stream);
-    case 3: return panel_waves<3>(x, x_stride, w, y, M, N, K, waves, stream);
-    default: return panel_waves<4>(x, x_stride, w, y, M, N, K, waves, stream);
+    case 1: return panel_waves<1>(x, x_stride, w, y, M, N, K, waves, stream, act);
+    case 2: return panel_waves<2>(x, x_stride, w, y, M, N, K, waves, stream, act);
+    case 3: return panel_waves<3>(x, x_stride, w, y, M, N, K, waves, stream, act);
+    default: return panel_waves<4>(x, x_stride, w, y, M, N, K, waves, stream, act);
   }
 }
 

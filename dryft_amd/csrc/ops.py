@@ -61,6 +61,7 @@ _SIGNATURES = {
              "dryft_gemm_stream_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_wide_bf16": [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
              "dryft_gemm_panel_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
+             "dryft_gemm_panel_glu_clamped_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _F, _F, _P],
              "dryft_gemm_panel_waves": [_I],
              "dryft_gemm_tall_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
              "dryft_gemm_tall_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -765,10 +766,11 @@ def gemm_panel_waves(n_outputs: int) -> int:
     return int(_fn("gemm", "dryft_gemm_panel_waves")(int(n_outputs)))
 
 
-def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
+def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0, clamped: tuple[float, float] | None = None) -> torch.Tensor:
     """``silu(x @ Wg.T) * (x @ Wu.T)`` for ``w_gate_up = [Wg; Wu]``, at most 64 rows, by the kernel whose operands go
     from memory straight into LDS. K must be a multiple of 128. ``waves`` (4 to 8, 8 outputs each) per workgroup;
-    0 lets the library choose."""
+    0 lets the library choose. ``clamped = (limit, alpha)``: the clamped gated unit in the epilogue instead,
+    ``g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(x @ Wg.T, limit)`` and ``u = clamp(x @ Wu.T, -limit, limit)``."""
     _gpu(x, "x", torch.bfloat16)
     _gpu(w_gate_up, "w_gate_up", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
@@ -784,6 +786,14 @@ def gemm_panel_swiglu_bf16(x, w_gate_up, out, waves: int = 0) -> torch.Tensor:
         raise KernelError(f"gemm_panel_swiglu: out must be [{m},{two_n // 2}]")
     if not (waves == 0 or 4 <= waves <= 8):
         raise KernelError("gemm_panel_swiglu: waves 4 to 8, or 0")
+    if clamped is not None:
+        limit, alpha = clamped
+        if not limit > 0:
+            raise KernelError(f"gemm_panel_swiglu: the clamp's limit must be positive, got {limit}")
+        _check(_fn("gemm", "dryft_gemm_panel_glu_clamped_bf16")(
+            _ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k, int(waves), float(limit), float(alpha),
+            _stream()), "gemm_panel_glu_clamped_bf16")
+        return out
     _check(_fn("gemm", "dryft_gemm_panel_swiglu_bf16")(_ptr(x), x.stride(0), _ptr(w_gate_up), _ptr(out), m, two_n // 2, k,
                                                        int(waves), _stream()), "gemm_panel_swiglu_bf16")
     return out

@@ -67,7 +67,11 @@ class ClampedGLU(FeedForward):
 
     def forward(self, h, ctx):
         act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
-        ops.glu_clamped(linear(h, self.w_gate_up), act, self.limit, self.alpha)
+        if h.dtype == torch.bfloat16 and panel_swiglu_ok(h, self.w_gate_up):
+            # up to 64 rows: product and unit in one kernel, the unit on the float accumulators
+            ops.gemm_panel_swiglu_bf16(h, self.w_gate_up, act, clamped=(self.limit, self.alpha))
+        else:
+            ops.glu_clamped(linear(h, self.w_gate_up), act, self.limit, self.alpha)
         return linear(act, self.w_down, allow_partials=True)
 
 

@@ -80,23 +80,26 @@ def test_stream_norm_every_combination(dtype, width):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_clamped_glu_part(dtype):
+@pytest.mark.parametrize("hidden", [72, 128, 256])
+def test_clamped_glu_part(dtype, hidden):
+    """``hidden`` 128 and 256: in bfloat16 steps of up to 64 rows take the product with the unit in its epilogue."""
     from dryft_amd.parts.base import Partials
     from dryft_amd.parts.mlp import ClampedGLU
     T = TORCH[dtype]
     g = torch.Generator().manual_seed(3)
-    w = {"gate": 2 * torch.randn(104, 72, generator=g) / 8, "up": 2 * torch.randn(104, 72, generator=g) / 8,
-         "down": torch.randn(72, 104, generator=g) / 10}
+    w = {"gate": 2 * torch.randn(104, hidden, generator=g) / hidden ** 0.5, "up": 2 * torch.randn(104, hidden, generator=g) / hidden ** 0.5,
+         "down": torch.randn(hidden, 104, generator=g) / 10}
     w = {k: v.to(T) for k, v in w.items()}
-    ffn = ClampedGLU(72, 104, limit=0.8)
+    ffn = ClampedGLU(hidden, 104, limit=0.8)
     ffn.load({k + "_proj": v.to(DEV) for k, v in w.items()})
-    for rows in (1, 9, 130):
-        h = torch.randn(rows, 72, generator=g).to(T)
+    for rows in (1, 9, 40, 130):
+        h = torch.randn(rows, hidden, generator=g).to(T)
         out = ffn.forward(h.to(DEV), None)
         if isinstance(out, Partials):
             out = out.summed(torch.float32)
         want = P.clamped_glu(h.double(), double(w), {"limit": 0.8})
         assert float((h.double() @ w["gate"].double().T).max()) > 0.8          # the clamp is at work
+        assert float((h.double() @ w["up"].double().T).min()) < -0.8
         assert rel_err(out, want) <= MIXER_TOL[dtype]
 
 
