@@ -175,6 +175,11 @@ ATTENTION_SHAPES = {
     "rot-full": dict(heads=8, kv_heads=1, dim=32, vdim=32, scale=0.2, softcap=50.0,
                      rot={"dims": 32, "base": 1e6, "scaling": None}),
     "bare": dict(heads=3, kv_heads=3, dim=20, vdim=12, scale=0.25, softcap=None, rot=None),
+    # the widths of real models' heads: half of each head rotated with scaled frequencies; a head of 64 without a cap
+    "head-128": dict(heads=4, kv_heads=2, dim=128, vdim=128, scale=128 ** -0.5, softcap=50.0,
+                     rot={"dims": 64, "base": 1e6, "scaling": {"factor": 8.0, "original": 128, "fast": 32.0, "slow": 1.0}}),
+    "head-64": dict(heads=2, kv_heads=2, dim=64, vdim=64, scale=0.125, softcap=None,
+                    rot={"dims": 64, "base": 10000.0, "scaling": None}),
 }
 
 
@@ -221,7 +226,9 @@ def test_attention_far_key_and_sink_show(dtype):
 
 
 MEMORY_SHAPES = {"narrow": dict(heads=2, dim=16, vdim=24, gate_cap=8.0), "one": dict(heads=1, dim=40, vdim=8, gate_cap=15.0),
-                 "wide": dict(heads=3, dim=24, vdim=72, gate_cap=12.0), "deep": dict(heads=1, dim=200, vdim=130, gate_cap=10.0)}
+                 "wide": dict(heads=3, dim=24, vdim=72, gate_cap=12.0), "deep": dict(heads=1, dim=200, vdim=130, gate_cap=10.0),
+                 # a real model's head: four runs of value columns, two tiles of key features a wave; and the widest key
+                 "head-128": dict(heads=2, dim=128, vdim=256, gate_cap=15.0), "key-256": dict(heads=1, dim=256, vdim=64, gate_cap=15.0)}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -267,7 +274,8 @@ def test_matrix_memory_keeps_an_early_token(dtype):
 
 
 RECURRENCE_SHAPES = {"three": dict(width=96, blocks=3, conv=3), "one-tap": dict(width=64, blocks=4, conv=1),
-                     "one-block": dict(width=72, blocks=1, conv=2), "five": dict(width=640, blocks=2, conv=5)}
+                     "one-block": dict(width=72, blocks=1, conv=2), "five": dict(width=640, blocks=2, conv=5),
+                     "blocks-128": dict(width=512, blocks=4, conv=4)}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
