@@ -555,6 +555,55 @@ __global__ __launch_bounds__(256) void rope_pairs_kv_kernel(const T* __restrict_
   for (int i = rot + lane; i < head_dim; i += WAVE) dst[i] = src[i];
 }
 
+// The same for steps of many rows whose widths come in 16-byte pieces (head width, rotated width and the columns
+// of q and k multiples of 8): a lane takes 8 neighbouring features of one q or k head, four pairs, with one load
+// and one store of 16 bytes and the pairs' four cosines and sines in two more. Values are not handled here.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_pairs_vec_kernel(const T* __restrict__ proj, int64_t proj_stride, int q_col,
+                                                             int k_col, const float* __restrict__ cos_t,
+                                                             const float* __restrict__ sin_t, int rot,
+                                                             const int* __restrict__ row_slot,
+                                                             const int* __restrict__ row_pos, T* __restrict__ q_out,
+                                                             T* __restrict__ k_pages,
+                                                             const int* __restrict__ page_table, int max_pages,
+                                                             int write_kv, int n_heads, int n_kv, int head_dim) {
+  const int lph = head_dim / 8;                         // lanes a head
+  const int64_t row = blockIdx.x;
+  const int idx = blockIdx.y * blockDim.x + threadIdx.x, job = idx / lph, part = idx % lph;
+  if (job >= n_heads + (write_kv ? n_kv : 0)) return;
+  const int slot = row_slot[row], pos = row_pos[row];
+  const bool is_q = job < n_heads;
+  T* dst;
+  if (is_q) {
+    dst = q_out + (row * n_heads + job) * head_dim + 8 * part;
+    if (slot < 0) {
+      const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      store8_from_float(dst, z);
+      return;
+    }
+  } else {
+    if (slot < 0) return;
+    const int page = page_of(page_table, max_pages, slot, pos);
+    if (page < 0) return;
+    dst = k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + pos % PAGE_TOKENS) * head_dim + 8 * part;
+  }
+  const T* src = proj + row * proj_stride + (is_q ? q_col + (int64_t)job * head_dim : k_col + (int64_t)(job - n_heads) * head_dim) +
+                 8 * part;
+  float v[8];
+  load8_as_float(src, v);
+  if (8 * part < rot) {                                 // rot is a multiple of 8: all four pairs turn, or none
+    const int half = rot / 2;
+    const vf4 c = *(const vf4*)(cos_t + (int64_t)pos * half + 4 * part), s = *(const vf4*)(sin_t + (int64_t)pos * half + 4 * part);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = v[2 * j], b = v[2 * j + 1];
+      v[2 * j] = a * c[j] - b * s[j];
+      v[2 * j + 1] = b * c[j] + a * s[j];
+    }
+  }
+  store8_from_float(dst, v);
+}
+
 DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_col, int k_col, int v_col,
                                   const float* cos_t, const float* sin_t, int rot, const int* row_slot,
                                   const int* row_pos, void* q_out, void* k_pages, void* v_pages,
@@ -567,7 +616,20 @@ DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_c
   const int skip_v = (write_kv && n_rows >= 32 && v_dim % 8 == 0 && v_col % 8 == 0 && proj_stride % 8 == 0 &&
                       (((uintptr_t)proj | (uintptr_t)v_pages) & 15) == 0 && v_lds <= 64 * 1024) ? 1 : 0;
   dim3 grid(n_rows, (n_heads + (skip_v ? 1 : 2) * n_kv + 3) / 4), block(256);
-  if (is_f32)
+  const bool vec = skip_v && head_dim % 8 == 0 && rot % 8 == 0 && q_col % 8 == 0 && k_col % 8 == 0 &&
+                   (((uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0;
+  if (vec) {
+    const int lanes = (n_heads + n_kv) * (head_dim / 8);
+    dim3 vg(n_rows, (lanes + 255) / 256);
+    if (is_f32)
+      hipLaunchKernelGGL(rope_pairs_vec_kernel<float>, vg, block, 0, stream, (const float*)proj, proj_stride, q_col, k_col,
+                         cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages, page_table, max_pages,
+                         write_kv, n_heads, n_kv, head_dim);
+    else
+      hipLaunchKernelGGL(rope_pairs_vec_kernel<bf16_t>, vg, block, 0, stream, (const bf16_t*)proj, proj_stride, q_col,
+                         k_col, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out, (bf16_t*)k_pages, page_table,
+                         max_pages, write_kv, n_heads, n_kv, head_dim);
+  } else if (is_f32)
     hipLaunchKernelGGL(rope_pairs_kv_kernel<float>, grid, block, 0, stream, (const float*)proj, proj_stride, q_col,
                        k_col, v_col, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages,
                        (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v);
