@@ -246,18 +246,19 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define CH_PAD 8
 #define CH_MAX_DT 4             // tiles of 16 key features a wave may own: D <= 256
 
-// Long prompts are also cut into segments of several chunks that run side by side, in two launches of this
-// kernel. MODE 1 walks every segment but a sequence's last from an empty memory (the first from the state the
-// step found, of which it also leaves a copy) and leaves what the segment makes of it: (S, n, m) and the sum B of
-// its log forget gates. Applying such a summary to a state (S_0, n_0, m_0) is m' = max(m_0 + B, m),
-// S' = exp(m_0 + B - m') S_0 + exp(m - m') S. MODE 2 folds the summaries before its segment into the state that
-// enters it, then walks its chunks as MODE 0 (one workgroup a sequence, no segments) does; a sequence's last
-// segment leaves the state. `tile_cu`: prefix sums over the sequences of their segments.
+// Long prompts are also cut into segments of several chunks that run side by side, in three launches. MODE 1 of
+// this kernel walks every segment but a sequence's last from an empty memory and leaves what the segment makes of
+// one: (S, n, m) and the sum B of its log forget gates. Applying such a summary to a state (S_0, n_0, m_0) is
+// m' = max(m_0 + B, m), S' = exp(m_0 + B - m') S_0 + exp(m - m') S. `mlstm_carry_kernel` does that from segment to
+// segment, starting from the state the step found, and leaves the state that enters each segment (the S part in the
+// summary's place). MODE 2 walks each segment from the state that enters it, as MODE 0 (one workgroup a sequence, no
+// segments) walks a whole sequence; a sequence's last segment leaves the state, which no other workgroup of that
+// launch reads. `tile_cu`: prefix sums over the sequences of their segments.
 struct Segments {
   const int* tile_cu;
   int n_seqs, seg_rows;
-  float *sum_s, *sum_n, *sum_m;       // [segments, heads, ...] as the state, and (m, B)
-  float *start_s, *start_n, *start_m; // [sequences, heads, ...]: the state the step found
+  float *sum_s, *sum_n, *sum_m;       // [segments, heads, ...] as the state, and (m, B); sum_s becomes the entering S
+  float *carry_n, *carry_m;           // [segments, heads, ...]: the n and m that enter each segment
 };
 
 template <int KB, int MODE>     // KB = ceil(D / 32)
@@ -293,7 +294,7 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   const int tok_first = MODE == 0 ? 0 : seg * sg.seg_rows;
   const int tok_end = MODE == 0 ? n_tok : min(n_tok, tok_first + sg.seg_rows);
   const bool last_seg = seg == n_segs - 1;
-  if (MODE == 1 && last_seg && seg > 0) return;                 // nobody folds a sequence's last segment
+  if (MODE == 1 && last_seg) return;                            // nobody folds a sequence's last segment
   bf16_t* k_s = (bf16_t*)lds_raw;                               // [64][KS]      keys, row-wise
   bf16_t* kw_t = k_s + CH_L * KS;                               // [DP][TS]      (w_s k_s)^T, positions permuted
   bf16_t* v_t = kw_t + DP * TS;                                 // [64][TS]      V^T, positions permuted
@@ -309,19 +310,18 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   float* N = state_n + (sh * gridDim.z + blockIdx.z) * dim;     // n and m: this run of value columns' own copy
   float* M_state = state_m + sh * gridDim.z + blockIdx.z;
   const int64_t per_s = (int64_t)dim * v_dim;
-  // where this workgroup's memory comes from: the state; in MODE 2 the copy MODE 1 left of it (a sequence of one
-  // segment reads the state itself: the workgroup that reads it is the one that writes it); nothing for a
-  // segment that MODE 1 walks from an empty memory; the first segment's summary for the later segments of MODE 2
+  // where this workgroup's memory comes from: the state (a sequence of one segment reads the state itself in MODE 2
+  // too: the workgroup that reads it is the one that writes it); nothing in MODE 1; in MODE 2 what the carry left
   const float* src_s = S;
   const float* src_n = N;
   const float* src_m = M_state;
   if (MODE == 2 && n_segs > 1) {
-    const int64_t at = seg == 0 ? (int64_t)seq * n_heads + head : (int64_t)seg_first * n_heads + head;
-    src_s = (seg == 0 ? sg.start_s : sg.sum_s) + at * per_s;
-    src_n = (seg == 0 ? sg.start_n : sg.sum_n) + at * dim;
-    src_m = seg == 0 ? sg.start_m + at : sg.sum_m + 2 * at;
+    const int64_t at = (int64_t)blockIdx.x * n_heads + head;
+    src_s = sg.sum_s + at * per_s;
+    src_n = sg.carry_n + at * dim;
+    src_m = sg.carry_m + at;
   }
-  const bool empty = MODE == 1 && seg > 0;
+  const bool empty = MODE == 1;
   // the state: S^T tiles [value tile vt][own key-feature tile j], d-tile index = wave + 4 j
   f32x4 acc_s[4][DT];
 #pragma unroll
@@ -338,48 +338,6 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   for (int d = threadIdx.x; d < DP; d += blockDim.x) n_s[d] = (!empty && d < dim) ? src_n[d] : 0.f;
   float m0 = empty ? -INFINITY : src_m[0];
   float b_sum = 0.f;
-  if (MODE == 1 && seg == 0) {                                  // the copy of the state the step found
-    const int64_t at = (int64_t)seq * n_heads + head;
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt)
-#pragma unroll
-      for (int j = 0; j < DT; ++j) {
-        const int d = 16 * (wave + 4 * j) + c;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int v = v0 + 16 * vt + 4 * g + i;
-          if (d < dim && v < v_dim) sg.start_s[at * per_s + (int64_t)d * v_dim + v] = acc_s[vt][j][i];
-        }
-      }
-    if (blockIdx.z == 0) {
-      for (int d = threadIdx.x; d < dim; d += blockDim.x) sg.start_n[at * dim + d] = src_n[d];
-      if (threadIdx.x == 0) sg.start_m[at] = m0;
-    }
-    if (last_seg) return;                                       // a sequence of one segment: MODE 2 does the rest
-  }
-  if (MODE == 2) {                                              // what the segments in between make of it
-    for (int k = 1; k < seg; ++k) {
-      const int64_t at = (int64_t)(seg_first + k) * n_heads + head;
-      const float mk = sg.sum_m[2 * at], bk = sg.sum_m[2 * at + 1];
-      const float m_new = fmaxf(m0 + bk, mk);
-      const float keep = expf(m0 + bk - m_new), take = expf(mk - m_new);
-      const float* ds = sg.sum_s + at * per_s;
-#pragma unroll
-      for (int vt = 0; vt < 4; ++vt)
-#pragma unroll
-        for (int j = 0; j < DT; ++j) {
-          const int d = 16 * (wave + 4 * j) + c;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int v = v0 + 16 * vt + 4 * g + i;
-            const float add = (d < dim && v < v_dim) ? ds[(int64_t)d * v_dim + v] : 0.f;
-            acc_s[vt][j][i] = keep * acc_s[vt][j][i] + take * add;
-          }
-        }
-      for (int d = threadIdx.x; d < dim; d += blockDim.x) n_s[d] = keep * n_s[d] + take * sg.sum_n[at * dim + d];
-      m0 = m_new;
-    }
-  }
   for (int t0 = tok_first; t0 < tok_end; t0 += CH_L) {
     const int nt = min(CH_L, tok_end - t0);
     __syncthreads();                                            // the chunk before is done with every buffer
@@ -583,6 +541,69 @@ __global__ __launch_bounds__(256) void mlstm_chunks_kernel(
   if (threadIdx.x == 0) M_state[0] = m0;
 }
 
+// From segment to segment: the state that enters each (see above). Grid (sequence, head, run of 64 value columns);
+// a thread keeps its elements of the run's slice of S in registers across the segments.
+#define CARRY_SPLIT 4            // workgroups that share a run's rows of S
+#define CARRY_HELD 16            // dim * 64 / 256 / CARRY_SPLIT for dim up to 256
+__global__ __launch_bounds__(256) void mlstm_carry_kernel(const int* __restrict__ seq_slot,
+                                                          const float* __restrict__ state_s,
+                                                          const float* __restrict__ state_n,
+                                                          const float* __restrict__ state_m, int n_heads, int dim,
+                                                          int v_dim, Segments sg) {
+  const int seq = blockIdx.x, head = blockIdx.y, run = blockIdx.z / CARRY_SPLIT, quarter = blockIdx.z % CARRY_SPLIT;
+  const int runs = gridDim.z / CARRY_SPLIT, v0 = run * CH_VS;
+  const int slot = seq_slot[seq];
+  if (slot < 0) return;
+  const int first = sg.tile_cu[seq], n_segs = sg.tile_cu[seq + 1] - first;
+  if (n_segs <= 1) return;
+  const int64_t sh = (int64_t)slot * n_heads + head, per_s = (int64_t)dim * v_dim;
+  const float* S = state_s + sh * per_s;
+  const int lane_v = threadIdx.x % CH_VS, d0 = threadIdx.x / CH_VS;      // element i of the thread: row 4 (d0 + 4 i) + quarter
+  const bool v_ok = v0 + lane_v < v_dim;
+  const bool writes_nm = run == 0 && quarter == 0;
+  float cur[CARRY_HELD];
+#pragma unroll
+  for (int i = 0; i < CARRY_HELD; ++i) {
+    const int d = 4 * (d0 + 4 * i) + quarter;
+    cur[i] = (d < dim && v_ok) ? S[(int64_t)d * v_dim + v0 + lane_v] : 0.f;
+  }
+  float n_cur = (int)threadIdx.x < dim ? state_n[(sh * runs + run) * dim + threadIdx.x] : 0.f;
+  float m_cur = state_m[sh * runs + run];
+  for (int j = 0; j < n_segs; ++j) {
+    const int64_t at = (int64_t)(first + j) * n_heads + head;
+    const bool more = j < n_segs - 1;                       // the last segment has no summary, and nothing after it
+    float keep = 1.f, take = 0.f, m_new = m_cur;
+    if (more) {
+      const float mk = sg.sum_m[2 * at], bk = sg.sum_m[2 * at + 1];
+      m_new = fmaxf(m_cur + bk, mk);
+      keep = expf(m_cur + bk - m_new);
+      take = expf(mk - m_new);
+    }
+    float* ss = sg.sum_s + at * per_s;
+    float add[CARRY_HELD];
+#pragma unroll
+    for (int i = 0; i < CARRY_HELD; ++i) {                  // all of the summary's values asked for before any is overwritten
+      const int d = 4 * (d0 + 4 * i) + quarter;
+      add[i] = (more && d < dim && v_ok) ? ss[(int64_t)d * v_dim + v0 + lane_v] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < CARRY_HELD; ++i) {
+      const int d = 4 * (d0 + 4 * i) + quarter;
+      if (d < dim && v_ok) {
+        ss[(int64_t)d * v_dim + v0 + lane_v] = cur[i];
+        cur[i] = keep * cur[i] + take * add[i];
+      }
+    }
+    if ((int)threadIdx.x < dim) {
+      const float more_n = more ? sg.sum_n[at * dim + threadIdx.x] : 0.f;
+      if (writes_nm) sg.carry_n[at * dim + threadIdx.x] = n_cur;
+      n_cur = keep * n_cur + take * more_n;
+    }
+    if (writes_nm && threadIdx.x == 0) sg.carry_m[at] = m_cur;
+    m_cur = m_new;
+  }
+}
+
 // Does the chunked kernel take these sizes? (16-byte pieces of rows; key width up to 256.)
 DRYFT_API int dryft_mlstm_chunks_takes(int dim, int v_dim, int q_col, int k_col, int v_col, int64_t proj_stride) {
   return dim > 0 && dim <= 64 * CH_MAX_DT && dim % 8 == 0 && v_dim % 8 == 0 && q_col % 8 == 0 && k_col % 8 == 0 &&
@@ -591,7 +612,7 @@ DRYFT_API int dryft_mlstm_chunks_takes(int dim, int v_dim, int q_col, int k_col,
 
 // seg_rows == 0: one workgroup walks a whole sequence. Otherwise (a multiple of 64): sequences are cut into
 // segments of that many rows, `tile_cu` holding the prefix sums of their counts and `max_tiles` a bound on their
-// total, and `scratch` room for the summaries: (max_tiles + n_seqs) * heads * (dim * v_dim + dim + 2) floats.
+// total, and `scratch` room for the summaries: max_tiles * heads * (dim * v_dim + 2 * dim + 3) floats.
 DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_col, int k_col, int v_col,
                                  const float* gates, const float* bias_i, const float* bias_f, float cap,
                                  const int* seq_slot, const int* cu_rows, const int* q_len, int n_seqs, float* state_s,
@@ -613,9 +634,8 @@ DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_co
     sg.sum_s = scratch;
     sg.sum_n = sg.sum_s + max_tiles * per;
     sg.sum_m = sg.sum_n + max_tiles * per_n;
-    sg.start_s = sg.sum_m + max_tiles * per_m * 2;
-    sg.start_n = sg.start_s + n_seqs * per;
-    sg.start_m = sg.start_n + n_seqs * per_n;
+    sg.carry_n = sg.sum_m + max_tiles * per_m * 2;
+    sg.carry_m = sg.carry_n + max_tiles * per_n;
   }
   const int vs = (v_dim + CH_VS - 1) / CH_VS;
 #define MC1(KBV, MODEV, GRIDX)                                                                                        \
@@ -629,7 +649,12 @@ DRYFT_API int dryft_mlstm_chunks(const void* proj, int64_t proj_stride, int q_co
                        state_m, o_raw, n_heads, dim, v_dim, q_scale, write_state, sg);                               \
   }
 #define MC(KBV)                                                                                                      \
-  if (seg_rows == 0) MC1(KBV, 0, n_seqs) else { MC1(KBV, 1, max_tiles) MC1(KBV, 2, max_tiles) }
+  if (seg_rows == 0) MC1(KBV, 0, n_seqs) else {                                                                      \
+    MC1(KBV, 1, max_tiles)                                                                                           \
+    hipLaunchKernelGGL(mlstm_carry_kernel, dim3(n_seqs, n_heads, vs * CARRY_SPLIT), dim3(256), 0, stream, seq_slot, state_s, \
+                       state_n, state_m, n_heads, dim, v_dim, sg);                                                   \
+    MC1(KBV, 2, max_tiles)                                                                                           \
+  }
   switch (kb) {
     case 1: MC(1); break;
     case 2: MC(2); break;

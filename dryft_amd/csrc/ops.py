@@ -1140,7 +1140,7 @@ def mlstm_steps(proj, q_col: int, k_col: int, v_col: int, gates, bias_i, bias_f,
             _gpu(tile_cu, "tile_cu", torch.int32)
             if not (tile_cu.is_contiguous() and tile_cu.numel() >= n_seqs + 1):
                 raise KernelError(f"tile_cu: needs {n_seqs + 1} contiguous entries")
-            scratch = torch.empty((max_tiles + n_seqs) * n_heads * (dim * v_dim + dim + 2), dtype=torch.float32,
+            scratch = torch.empty(max_tiles * n_heads * (dim * v_dim + 2 * dim + 3), dtype=torch.float32,
                                   device=proj.device)
         _check(_fn("mlstm", "dryft_mlstm_chunks")(
             _ptr(proj), proj.stride(0), q_col, k_col, v_col, _ptr(gates), _ptr(bias_i), _ptr(bias_f), float(cap),
