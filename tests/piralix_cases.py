@@ -131,3 +131,34 @@ def variant(cfg: dict, **changes) -> dict:
     out = copy.deepcopy(cfg)
     out.update(changes)
     return out
+
+
+def random_config(rng) -> dict:
+    """A configuration drawn with ``rng`` (a ``random.Random``): sizes, head counts, the order of layers, where
+    feed-forwards sit, what is rotated and how, caps, taps, blocks and the loop all vary."""
+    width = rng.choice([64, 96, 128, 160, 192, 256, 320])
+    vocab = rng.randrange(100, 600)
+    layers = []
+    for _ in range(rng.randrange(3, 7)):
+        kind = rng.choice(["attention", "mlstm", "rglru"])
+        if kind == "attention":
+            kv = rng.choice([1, 2, 4])
+            heads = kv * rng.choice([1, 2, 3, 4])
+            dim = rng.choice([16, 24, 32, 48, 64, 80, 128])
+            vdim = rng.choice([dim, dim, 16, 40, 64])
+            rot = rng.choice([None, dim, (dim // 4) * 2, 8])
+            scaling = rng.choice([None, SCALING, {"factor": 2.0, "original": 32, "fast": 16.0, "slow": 2.0}]) if rot else None
+            layer = attention(heads, kv, dim, vdim, rot_dims=rot, base=rng.choice([500.0, 1e4, 1e6]), scaling=scaling,
+                              softcap=rng.choice([None, 10.0, 30.0, 50.0]), scale=rng.choice([dim ** -0.5, 0.2, 0.05]))
+        elif kind == "mlstm":
+            layer = mlstm(rng.choice([1, 2, 4, 5]), rng.choice([16, 32, 48, 64, 96, 128]),
+                          rng.choice([16, 24, 32, 64, 72, 128, 136]), cap=rng.choice([6.0, 12.0, 20.0]))
+        else:
+            blocks, block = rng.choice([1, 2, 4, 8]), rng.choice([8, 16, 32, 40, 64, 96])
+            layer = rglru(blocks * block, blocks, rng.choice([1, 2, 3, 4, 6]))
+        layers.append(with_mlp(layer, ff=rng.choice([None, 48, 128, 200, 256]), limit=rng.choice([0.75, 1.5, 7.0])))
+    loop = None
+    if rng.random() < 0.75:
+        start = rng.randrange(0, len(layers))
+        loop = {"start": start, "stop": rng.randrange(start + 1, len(layers) + 1), "times": rng.choice([1, 2, 2, 3])}
+    return config(width, vocab, layers, loop=loop, eps=rng.choice([1e-6, 1e-5]))
