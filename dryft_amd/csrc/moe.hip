@@ -1,0 +1,309 @@
+// Routed experts on the device: the router's choice, the sort of (row, expert) pairs by expert, the grouped
+// products over each expert's rows, and the weighted sum per row. No step of it needs the host, so a step that
+// holds it can be captured.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 512
+#define MOE_PER_LANE (MOE_MAX_EXPERTS / WAVE)
+#define MOE_TILE 32            // pairs of one expert that a workgroup of the products takes
+
+struct Best {
+  float v;
+  int i;
+};
+
+// The larger value; of equal values the lower index.
+__device__ __forceinline__ Best wave_best(Best b) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    const float v = __shfl_xor(b.v, o, WAVE);
+    const int i = __shfl_xor(b.i, o, WAVE);
+    if (v > b.v || (v == b.v && i < b.i)) { b.v = v; b.i = i; }
+  }
+  return b;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Router. s = sigmoid(z); choice = s + correction. Experts form `groups` equal groups of neighbours; a group's
+// score is the sum of its two largest choice scores (of its only one, if it has one); experts outside the `keep`
+// best groups drop out. The `top` largest choice scores that remain are chosen, highest first, and weigh
+// s / (sum of the chosen s + 1e-20) * scale. One wave a row; lane l holds experts l, l + 64, ...
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int64_t stride,
+                                                        const float* __restrict__ correction, int n_experts, int groups,
+                                                        int keep, int top, float scale, int* __restrict__ chosen,
+                                                        float* __restrict__ weights, int rows) {
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  const float NEG = -__builtin_inff();
+  float s[MOE_PER_LANE], c[MOE_PER_LANE];
+#pragma unroll
+  for (int j = 0; j < MOE_PER_LANE; ++j) {
+    const int e = lane + WAVE * j;
+    s[j] = 0.f;
+    c[j] = NEG;
+    if (e < n_experts) {
+      s[j] = 1.f / (1.f + expf(-logits[row * stride + e]));
+      c[j] = s[j] + correction[e];
+    }
+  }
+  if (keep < groups) {
+    const int size = n_experts / groups;
+    float score = NEG;               // lane g holds group g's score
+    for (int g = 0; g < groups; ++g) {
+      Best a{NEG, 0x7fffffff};
+#pragma unroll
+      for (int j = 0; j < MOE_PER_LANE; ++j) {
+        const int e = lane + WAVE * j;
+        if (e < n_experts && e / size == g && (c[j] > a.v || (c[j] == a.v && e < a.i))) { a.v = c[j]; a.i = e; }
+      }
+      a = wave_best(a);
+      float sum = a.v;
+      if (size >= 2) {
+        Best b{NEG, 0x7fffffff};
+#pragma unroll
+        for (int j = 0; j < MOE_PER_LANE; ++j) {
+          const int e = lane + WAVE * j;
+          if (e < n_experts && e / size == g && e != a.i && (c[j] > b.v || (c[j] == b.v && e < b.i))) { b.v = c[j]; b.i = e; }
+        }
+        b = wave_best(b);
+        sum += b.v;
+      }
+      if (lane == g) score = sum;
+    }
+    uint64_t kept = 0;
+    for (int i = 0; i < keep; ++i) {
+      Best a{(lane < groups && !((kept >> lane) & 1)) ? score : NEG, lane < groups ? lane : 0x7fffffff};
+      if (lane < groups && ((kept >> lane) & 1)) a.i = 0x7fffffff;
+      a = wave_best(a);
+      if (a.i < groups) kept |= 1ull << a.i;
+    }
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      const int e = lane + WAVE * j;
+      if (e < n_experts && !((kept >> (e / size)) & 1)) c[j] = NEG;
+    }
+  }
+  float total = 0.f;
+  for (int i = 0; i < top; ++i) {
+    Best a{NEG, 0x7fffffff};
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j) {
+      const int e = lane + WAVE * j;
+      if (e < n_experts && (c[j] > a.v || (c[j] == a.v && e < a.i))) { a.v = c[j]; a.i = e; }
+    }
+    a = wave_best(a);
+    float sv = 0.f;
+#pragma unroll
+    for (int j = 0; j < MOE_PER_LANE; ++j)
+      if (lane + WAVE * j == a.i) { sv = s[j]; c[j] = NEG; }
+    sv = wave_sum(sv);
+    total += sv;
+    if (lane == 0) {
+      chosen[row * top + i] = a.i;
+      weights[row * top + i] = sv;       // divided below
+    }
+  }
+  if (lane == 0)       // the same lane wrote them
+    for (int i = 0; i < top; ++i) weights[row * top + i] = weights[row * top + i] / (total + 1e-20f) * scale;
+}
+
+DRYFT_API int dryft_moe_max_experts() { return MOE_MAX_EXPERTS; }
+DRYFT_API int dryft_moe_tile() { return MOE_TILE; }
+
+DRYFT_API int dryft_moe_route(const float* logits, int64_t stride, const float* correction, int n_experts, int groups,
+                              int keep, int top, float scale, int* chosen, float* weights, int rows, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (n_experts < 1 || n_experts > MOE_MAX_EXPERTS || top < 1 || top > n_experts || groups < 1 || groups > WAVE ||
+      n_experts % groups || keep < 1 || keep > groups || keep * (n_experts / groups) < top)
+    return -1;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, logits, stride, correction, n_experts,
+                     groups, keep, top, scale, chosen, weights, rows);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The plan of a step: pairs (row, k) sorted by expert (`sorted_pair`: place -> pair, `place_of`: pair -> place),
+// every expert's run of places cut into tiles of MOE_TILE. One workgroup. Which place a pair gets within its
+// expert's run depends on the order in which threads arrive; no result depends on it, since every pair's
+// outputs are computed from its own row alone, in a fixed order.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int n_pairs, int n_experts,
+                                                        int* __restrict__ sorted_pair, int* __restrict__ place_of,
+                                                        int* __restrict__ tile_expert, int* __restrict__ tile_start,
+                                                        int* __restrict__ tile_rows, int* __restrict__ n_tiles,
+                                                        int max_tiles) {
+  __shared__ int counts[MOE_MAX_EXPERTS], cursor[MOE_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&counts[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      cursor[e] = at;
+      for (int s = 0; s < counts[e] && nt < max_tiles; s += MOE_TILE) {
+        tile_expert[nt] = e;
+        tile_start[nt] = at + s;
+        tile_rows[nt] = min(MOE_TILE, counts[e] - s);
+        ++nt;
+      }
+      at += counts[e];
+    }
+    *n_tiles = nt;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+    const int place = atomicAdd(&cursor[chosen[p]], 1);
+    sorted_pair[place] = p;
+    place_of[p] = place;
+  }
+}
+
+DRYFT_API int dryft_moe_plan(const int* chosen, int n_pairs, int n_experts, int* sorted_pair, int* place_of,
+                             int* tile_expert, int* tile_start, int* tile_rows, int* n_tiles, int max_tiles,
+                             hipStream_t stream) {
+  if (n_pairs <= 0) return 0;
+  if (n_experts < 1 || n_experts > MOE_MAX_EXPERTS) return -1;
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, stream, chosen, n_pairs, n_experts, sorted_pair, place_of,
+                     tile_expert, tile_start, tile_rows, n_tiles, max_tiles);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Grouped product, plain multiply-adds: for every tile of an expert's places, out[place] = W_e a[place]. A
+// workgroup takes one tile (up to 32 places) and 64 outputs; K goes through LDS 32 at a time; a thread owns two
+// places and four outputs. With `top` > 0 the operand rows are gathered: place -> pair -> row pair / top of `a`;
+// otherwise `a` is already in place order. GLU: W_e holds gate rows then up rows; the clamped gated unit
+// g * sigmoid(alpha g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit), is applied to the float
+// accumulators and `n_out` counts its outputs.
+#define MOE_TN 64
+#define MOE_TK 32
+
+template <typename T, typename O, bool GLU>
+__global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ a, int64_t a_stride,
+                                                          const T* __restrict__ w, const int* __restrict__ sorted_pair,
+                                                          const int* __restrict__ tile_expert,
+                                                          const int* __restrict__ tile_start,
+                                                          const int* __restrict__ tile_rows,
+                                                          const int* __restrict__ n_tiles, O* __restrict__ out, int top,
+                                                          int n_out, int k_dim, float limit, float alpha) {
+  __shared__ float sa[MOE_TILE][MOE_TK + 1];
+  __shared__ float sw[(GLU ? 2 : 1) * MOE_TN][MOE_TK + 1];
+  __shared__ int src_row[MOE_TILE];
+  const int tile = blockIdx.x;
+  if (tile >= *n_tiles) return;
+  const int expert = tile_expert[tile], start = tile_start[tile], count = tile_rows[tile];
+  const int n0 = blockIdx.y * MOE_TN;
+  const int w_rows = GLU ? 2 * n_out : n_out;
+  const T* we = w + (int64_t)expert * w_rows * k_dim;
+  if (threadIdx.x < MOE_TILE)
+    src_row[threadIdx.x] = threadIdx.x < count ? (top > 0 ? sorted_pair[start + threadIdx.x] / top : start + threadIdx.x) : -1;
+  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;      // places ty, ty + 16; outputs tx + 16 j
+  float acc[2][4], acc_up[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = acc_up[i][j] = 0.f;
+  for (int k0 = 0; k0 < k_dim; k0 += MOE_TK) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < MOE_TILE * MOE_TK; e += 256) {
+      const int r = e / MOE_TK, kk = e % MOE_TK;
+      const int row = src_row[r];
+      sa[r][kk] = (row >= 0 && k0 + kk < k_dim) ? load_as_float(a + (int64_t)row * a_stride + k0 + kk) : 0.f;
+    }
+    for (int e = threadIdx.x; e < (GLU ? 2 : 1) * MOE_TN * MOE_TK; e += 256) {
+      const int r = e / MOE_TK, kk = e % MOE_TK;
+      const int n = n0 + r % MOE_TN;
+      const int64_t w_row = (GLU && r >= MOE_TN) ? (int64_t)n_out + n : n;
+      sw[r][kk] = (n < n_out && k0 + kk < k_dim) ? load_as_float(we + w_row * k_dim + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < MOE_TK; ++kk) {
+      const float a0 = sa[ty][kk], a1 = sa[ty + 16][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float b = sw[tx + 16 * j][kk];
+        acc[0][j] += a0 * b;
+        acc[1][j] += a1 * b;
+        if (GLU) {
+          const float u = sw[MOE_TN + tx + 16 * j][kk];
+          acc_up[0][j] += a0 * u;
+          acc_up[1][j] += a1 * u;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int r = ty + 16 * i;
+    if (r >= count) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx + 16 * j;
+      if (n >= n_out) continue;
+      float v = acc[i][j];
+      if (GLU) {
+        // the unit reads what the products would have stored in the activation dtype
+        const float g = fminf(rounded_as<T>(v), limit);
+        const float u = fminf(fmaxf(rounded_as<T>(acc_up[i][j]), -limit), limit);
+        v = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+      }
+      store_from_float(out + (int64_t)(start + r) * n_out + n, v);
+    }
+  }
+}
+
+DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, const int* sorted_pair,
+                                const int* tile_expert, const int* tile_start, const int* tile_rows, const int* n_tiles,
+                                int max_tiles, void* out, int out_is_f32, int top, int n_out, int k_dim, int glu,
+                                float limit, float alpha, int is_f32, hipStream_t stream) {
+  if (max_tiles <= 0) return 0;
+  if (n_out <= 0 || k_dim <= 0 || (glu && out_is_f32 && !is_f32)) return -1;
+  dim3 grid(max_tiles, (n_out + MOE_TN - 1) / MOE_TN), block(256);
+#define MOE_LAUNCH(T, O, G)                                                                                       \
+  hipLaunchKernelGGL((moe_product_kernel<T, O, G>), grid, block, 0, stream, (const T*)a, a_stride, (const T*)w,   \
+                     sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha)
+  if (is_f32) {
+    if (glu) MOE_LAUNCH(float, float, true); else MOE_LAUNCH(float, float, false);
+  } else if (glu) {
+    MOE_LAUNCH(bf16_t, bf16_t, true);
+  } else if (out_is_f32) {
+    MOE_LAUNCH(bf16_t, float, false);
+  } else {
+    MOE_LAUNCH(bf16_t, bf16_t, false);
+  }
+#undef MOE_LAUNCH
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// out[row] = sum_k weights[row, k] * y[place_of[row * top + k]]  (k in order)  + sigmoid(z_shared[row]) * shared[row]
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place_of,
+                                                          const float* __restrict__ weights, const T* __restrict__ shared,
+                                                          const float* __restrict__ logits, int64_t logit_stride,
+                                                          int shared_col, T* __restrict__ out, int top, int width) {
+  const int64_t row = blockIdx.x;
+  const float gate = shared ? 1.f / (1.f + expf(-logits[row * logit_stride + shared_col])) : 0.f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k)
+      acc += weights[row * top + k] * y[(int64_t)place_of[row * top + k] * width + c];
+    if (shared) acc += gate * load_as_float(shared + row * width + c);
+    store_from_float(out + row * width + c, acc);
+  }
+}
+
+DRYFT_API int dryft_moe_combine(const float* y, const int* place_of, const float* weights, const void* shared,
+                                const float* logits, int64_t logit_stride, int shared_col, void* out, int rows, int top,
+                                int width, int is_f32, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (is_f32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(rows), dim3(256), 0, stream, y, place_of, weights,
+                       (const float*)shared, logits, logit_stride, shared_col, (float*)out, top, width);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, y, place_of, weights,
+                       (const bf16_t*)shared, logits, logit_stride, shared_col, (bf16_t*)out, top, width);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -72,6 +72,19 @@ _SIGNATURES = {
              "dryft_gemm_rows_f32": [_P, _L, _P, _P, _I, _I, _I, _P],
              "dryft_gemm_wide_swiglu_bf16": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
              "dryft_sum_partials": [_P, _P, _L, _I, _I, _P]},
+    "hyper": {"dryft_hyper_norm": [_P, _I, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
+    "wkv": {"dryft_wkv_blend": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+            "dryft_wkv_decay": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
+            "dryft_wkv_steps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "dryft_wkv_out": [_P, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
+    "latent": {"dryft_rms_segments": [_P, _L, _I, _P, _P, _I, _P, _P, _I, _F, _I, _I, _P],
+               "dryft_latent_rope_kv": [_P, _P, _P, _L, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                        _I, _I, _I, _P],
+               "dryft_head_gate": [_P, _P, _L, _I, _P, _I, _I, _I, _I, _I, _P]},
+    "moe": {"dryft_moe_route": [_P, _L, _P, _I, _I, _I, _I, _F, _P, _P, _I, _P],
+            "dryft_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
+            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I, _P],
+            "dryft_moe_combine": [_P, _P, _P, _P, _P, _L, _I, _P, _I, _I, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _I, _P, _P, _P]},
 }
@@ -1286,3 +1299,336 @@ def rglru_scan_tiles(coef, proj, x_col: int, y_col: int, x_bias, y_bias, taps: i
         _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), _ptr(tile_cu), n_seqs, max_tiles, _ptr(state),
         _ptr(tail) if taps > 1 else 0, _ptr(out), width, int(bool(write_state)), _float_flag(proj, "proj"), _stream()),
         "rglru_scan_tiles")
+
+
+# ------------------------------------------------------------------------------------------ several copies of a stream
+HYPER_MAX_STREAMS = 8
+
+
+def hyper_norm(x, n: int, delta, mix, write, read, weight, eps: float, x_out, y, *, normed: bool) -> None:
+    """One launch for a residual stream of ``n`` copies: ``x'_t = sum_s mix[s, t] x_s + write[t] * delta`` (skipped
+    without ``delta``), written to ``x_out [n, rows, width]`` (float32, may be ``x``; None: not kept);
+    ``u = sum_t read[t] x'_t`` (``read`` None: the plain sum); ``y = rmsnorm(u) * weight`` in the activation dtype
+    when ``normed``, else ``y = u`` in float32. ``x`` is the copies in float32 or one ``[rows, width]`` tensor in the
+    activation dtype that every copy equals; ``delta`` a tensor in the activation dtype or ``(partials, count)``."""
+    _gpu(x, "x")
+    rows, width = x.shape[-2:]
+    copies = x.dim() == 3
+    if copies:
+        if not (x.dtype == torch.float32 and x.shape[0] == n and x.is_contiguous()):
+            raise KernelError(f"hyper_norm: the copies must be contiguous float32 [{n}, rows, width]")
+    elif not (x.dim() == 2 and x.is_contiguous()):
+        raise KernelError("hyper_norm: a stream that starts must be contiguous [rows, width]")
+    if not 1 <= n <= HYPER_MAX_STREAMS:
+        raise KernelError(f"hyper_norm: 1..{HYPER_MAX_STREAMS} copies, got {n}")
+    act = y.dtype if (y is not None and normed) else (x.dtype if not copies else None)
+    kind, n_partials, stride = 0, 0, 0
+    if delta is not None:
+        data, n_partials = delta if isinstance(delta, tuple) else (delta, 1)
+        _gpu(data, "delta")
+        if isinstance(delta, tuple):
+            if not (data.dtype == torch.float32 and data.dim() == 3 and data.shape[1:] == (rows, width) and
+                    data.is_contiguous() and data.shape[0] >= n_partials >= 1):
+                raise KernelError("hyper_norm: partial sums must be contiguous float32 [n, rows, width]")
+            kind, stride = 2, rows * width
+        else:
+            if not (data.shape == (rows, width) and data.is_contiguous()):
+                raise KernelError("hyper_norm: delta must be contiguous [rows, width]")
+            if act is None:
+                act = data.dtype
+            if data.dtype != act:
+                raise KernelError("hyper_norm: delta must be in the activation dtype")
+            kind = 1
+        delta = data
+        _f32_vector(mix, "mix", n * n)
+        _f32_vector(write, "write", n)
+    if act is None:
+        act = torch.float32
+    if not copies and x.dtype != act:
+        raise KernelError("hyper_norm: a stream that starts must be in the activation dtype")
+    if read is not None:
+        _f32_vector(read, "read", n)
+    if x_out is not None:
+        _gpu(x_out, "x_out", torch.float32)
+        if not (x_out.shape == (n, rows, width) and x_out.is_contiguous()):
+            raise KernelError("hyper_norm: x_out must be contiguous float32 [n, rows, width]")
+    if y is not None:
+        _gpu(y, "y", act if normed else torch.float32)
+        if not (y.shape == (rows, width) and y.is_contiguous()):
+            raise KernelError("hyper_norm: y must be contiguous [rows, width]")
+        if normed:
+            _f32_vector(weight, "weight", width)
+    _check(_fn("hyper", "dryft_hyper_norm")(
+        _ptr(x), int(copies), n, _ptr(delta), kind, n_partials, stride, _ptr(mix), _ptr(write), _ptr(read), _ptr(weight),
+        _ptr(x_out), _ptr(y), int(bool(normed)), rows, width, float(eps), 1 if act == torch.float32 else 0, _stream()),
+        "hyper_norm")
+
+
+# ------------------------------------------------------------------------------------------ wkv
+WKV_MAX_DIM = 256
+
+
+def wkv_blend(h, previous, mu, row_slot, row_seq, row_pos, seq_start, out) -> None:
+    """``out[b] = h + (h' - h) * mu[b]`` for the five blends, ``h'`` the row before of the same sequence
+    (``previous[slot]`` for a sequence's first row of the step)."""
+    _gpu(h, "h")
+    rows, width = h.shape
+    _gpu(out, "out", h.dtype)
+    _gpu(previous, "previous", torch.float32)
+    if not (h.is_contiguous() and out.shape == (5, rows, width) and out.is_contiguous()):
+        raise KernelError("wkv_blend: h contiguous [rows, width], out contiguous [5, rows, width]")
+    if not (previous.dim() == 2 and previous.shape[1] == width and previous.is_contiguous()):
+        raise KernelError("wkv_blend: previous must be contiguous float32 [slots, width]")
+    _f32_vector(mu, "mu", 5 * width)
+    for name, t in (("row_slot", row_slot), ("row_seq", row_seq), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        if t.numel() < rows:
+            raise KernelError(f"{name}: needs {rows} entries")
+    _gpu(seq_start, "seq_start", torch.int32)
+    _check(_fn("wkv", "dryft_wkv_blend")(_ptr(h), _ptr(previous), _ptr(mu), _ptr(row_slot), _ptr(row_seq), _ptr(row_pos),
+                                         _ptr(seq_start), _ptr(out), rows, width, _float_flag(h, "h"), _stream()),
+           "wkv_blend")
+
+
+def wkv_decay(low, up, bias, log_w) -> None:
+    """``log_w = -exp(tanh(low) @ up.T + bias)``: ``low`` float32 ``[rows, rank]``, ``up`` ``[n, rank]``."""
+    _gpu(low, "low", torch.float32)
+    _gpu(up, "up")
+    rows, rank = low.shape
+    n = up.shape[0]
+    if not (low.is_contiguous() and up.is_contiguous() and up.shape == (n, rank)):
+        raise KernelError(f"wkv_decay: low contiguous [rows, {rank}], up contiguous [n, {rank}], got {tuple(up.shape)}")
+    _f32_vector(bias, "bias", n)
+    _gpu(log_w, "log_w", torch.float32)
+    if not (log_w.shape == (rows, n) and log_w.is_contiguous()):
+        raise KernelError("wkv_decay: log_w must be contiguous float32 [rows, n]")
+    _check(_fn("wkv", "dryft_wkv_decay")(_ptr(low), _ptr(up), _ptr(bias), _ptr(log_w), rows, n, rank,
+                                         _float_flag(up, "up"), _stream()), "wkv_decay")
+
+
+def wkv_steps(r, k, v, log_w, bonus, seq_slot, cu_rows, q_len, n_seqs: int, state, o_raw, h, previous, n_heads: int,
+              dim: int, write_state: bool) -> None:
+    """The recurrence over every sequence's rows in order, from ``state[slot]`` (float32 ``[slots, heads, dim, dim]``)
+    to the raw read-outs ``o_raw`` (float32 ``[rows, heads * dim]``); when ``write_state`` the state is written back
+    and ``previous[slot]`` receives the sequence's last row of ``h``."""
+    _gpu(r, "r")
+    rows = r.shape[0]
+    inner = n_heads * dim
+    for name, t in (("r", r), ("k", k), ("v", v)):
+        _gpu(t, name, r.dtype)
+        if not (t.shape == (rows, inner) and t.is_contiguous()):
+            raise KernelError(f"wkv_steps: {name} must be contiguous [rows, {inner}]")
+    for name, t in (("log_w", log_w), ("o_raw", o_raw)):
+        _gpu(t, name, torch.float32)
+        if not (t.shape == (rows, inner) and t.is_contiguous()):
+            raise KernelError(f"wkv_steps: {name} must be contiguous float32 [rows, {inner}]")
+    _f32_vector(bonus, "bonus", inner)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(state, "state", torch.float32)
+    if not (state.dim() == 4 and state.shape[1:] == (n_heads, dim, dim) and state.is_contiguous()):
+        raise KernelError(f"wkv_steps: state must be contiguous float32 [slots, {n_heads}, {dim}, {dim}]")
+    _gpu(h, "h", r.dtype)
+    _gpu(previous, "previous", torch.float32)
+    if not (h.dim() == 2 and h.shape[0] == rows and h.is_contiguous() and previous.dim() == 2 and
+            previous.shape == (state.shape[0], h.shape[1]) and previous.is_contiguous()):
+        raise KernelError("wkv_steps: h contiguous [rows, width], previous contiguous float32 [slots, width]")
+    if not 0 < dim <= WKV_MAX_DIM:
+        raise KernelError(f"wkv_steps: dim must lie in 1..{WKV_MAX_DIM}")
+    _check(_fn("wkv", "dryft_wkv_steps")(
+        _ptr(r), _ptr(k), _ptr(v), _ptr(log_w), _ptr(bonus), _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs,
+        _ptr(state), _ptr(o_raw), _ptr(h), _ptr(previous), h.shape[1], n_heads, dim, int(bool(write_state)),
+        _float_flag(r, "r"), _stream()), "wkv_steps")
+
+
+def wkv_out(o_raw, gate, weight, out, n_heads: int, dim: int, eps: float) -> None:
+    """``out = o_raw / rms_per_head(o_raw) * weight * silu(gate)`` in the activation dtype."""
+    _gpu(gate, "gate")
+    rows = gate.shape[0]
+    inner = n_heads * dim
+    _gpu(o_raw, "o_raw", torch.float32)
+    _gpu(out, "out", gate.dtype)
+    for name, t in (("o_raw", o_raw), ("gate", gate), ("out", out)):
+        if not (t.shape == (rows, inner) and t.is_contiguous()):
+            raise KernelError(f"wkv_out: {name} must be contiguous [rows, {inner}]")
+    _f32_vector(weight, "weight", inner)
+    _check(_fn("wkv", "dryft_wkv_out")(_ptr(o_raw), _ptr(gate), _ptr(weight), _ptr(out), rows, n_heads, dim, float(eps),
+                                       _float_flag(gate, "gate"), _stream()), "wkv_out")
+
+
+# ------------------------------------------------------------------------------------------ latent attention
+def rms_segments(src, col: int, w_a, out_a, n_a: int, w_b, out_b, eps: float) -> None:
+    """``out_a = rmsnorm(src[:, col : col + n_a]) * w_a`` and, when ``out_b`` is given, the same for the columns
+    after them with ``w_b``; float statistics, plain float32 weights."""
+    _gpu(src, "src")
+    rows = src.shape[0]
+    n_b = out_b.shape[1] if out_b is not None else 0
+    if not (src.dim() == 2 and src.stride(1) == 1 and 0 <= col and col + n_a + n_b <= src.shape[1]):
+        raise KernelError("rms_segments: the runs of columns lie outside src")
+    for name, t, n, w in (("out_a", out_a, n_a, w_a), ("out_b", out_b, n_b, w_b)):
+        if t is None:
+            continue
+        _gpu(t, name, src.dtype)
+        if not (t.shape == (rows, n) and t.is_contiguous()):
+            raise KernelError(f"rms_segments: {name} must be contiguous [rows, {n}]")
+        _f32_vector(w, name + "'s weight", n)
+    _check(_fn("latent", "dryft_rms_segments")(_ptr(src), src.stride(0), col, _ptr(w_a), _ptr(out_a), n_a, _ptr(w_b),
+                                               _ptr(out_b), n_b, float(eps), rows, _float_flag(src, "src"), _stream()),
+           "rms_segments")
+
+
+def latent_rope_kv(q_raw, kv, down, krot_col: int, cos, sin, rot: int, row_slot, row_pos, q_out, k_pages, v_pages,
+                   page_table, write_kv: bool, n_heads: int, plain: int, rot_dim: int, v_dim: int, page_dv: int) -> None:
+    """Queries ``[plain | rotated]`` per head from ``q_raw``; keys ``[that head's plain part of kv | the one rotated
+    part at column krot_col of down]``; values from ``kv`` after the keys. The rotated parts' first ``rot`` features
+    turn, feature ``i`` with ``i + rot/2``, with float32 tables; keys and values go to their pages (values ``page_dv``
+    wide, of which ``v_dim`` are written)."""
+    _gpu(q_raw, "q_raw")
+    is_f32 = _float_flag(q_raw, "q_raw")
+    rows, key_dim = q_raw.shape[0], plain + rot_dim
+    if not (q_raw.shape == (rows, n_heads * key_dim) and q_raw.is_contiguous()):
+        raise KernelError(f"latent_rope_kv: q_raw must be contiguous [rows, {n_heads * key_dim}]")
+    _gpu(kv, "kv", q_raw.dtype)
+    if not (kv.shape == (rows, n_heads * (plain + v_dim)) and kv.is_contiguous()):
+        raise KernelError(f"latent_rope_kv: kv must be contiguous [rows, {n_heads * (plain + v_dim)}]")
+    _gpu(down, "down", q_raw.dtype)
+    if not (down.dim() == 2 and down.shape[0] == rows and down.stride(1) == 1 and 0 <= krot_col and
+            krot_col + rot_dim <= down.shape[1]):
+        raise KernelError("latent_rope_kv: the rotated key part lies outside down's columns")
+    if rot % 2 or not 0 <= rot <= rot_dim:
+        raise KernelError(f"latent_rope_kv: the rotated width must be even and at most {rot_dim}, got {rot}")
+    if rot:
+        for name, t in (("cos", cos), ("sin", sin)):
+            _gpu(t, name, torch.float32)
+            if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+                raise KernelError(f"{name}: must be contiguous float32 [positions, {rot // 2}]")
+    _gpu(q_out, "q_out", q_raw.dtype)
+    if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * key_dim):
+        raise KernelError("latent_rope_kv: q_out must be [rows, heads, key_dim]")
+    if not v_dim <= page_dv:
+        raise KernelError("latent_rope_kv: the values' pages are narrower than the values")
+    _check_pages(k_pages, v_pages, page_table, n_heads, key_dim, q_raw.dtype, page_dv)
+    for name, t in (("row_slot", row_slot), ("row_pos", row_pos)):
+        _gpu(t, name, torch.int32)
+        if not (t.numel() >= rows):
+            raise KernelError(f"{name}: needs {rows} entries")
+    _check(_fn("latent", "dryft_latent_rope_kv")(
+        _ptr(q_raw), _ptr(kv), _ptr(down), down.stride(0), krot_col, _ptr(cos), _ptr(sin), rot, _ptr(row_slot),
+        _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1],
+        int(bool(write_kv)), rows, n_heads, plain, rot_dim, v_dim, page_dv, is_f32, _stream()), "latent_rope_kv")
+
+
+def head_gate(attn, down, g_col: int, out, n_heads: int, v_dim: int) -> None:
+    """``out[row, head, :] = attn[row, head, :v_dim] * sigmoid(down[row, g_col + head])``; ``attn``'s heads may be
+    wider than ``v_dim``, ``out`` is packed ``[rows, heads * v_dim]``."""
+    _gpu(attn, "attn")
+    rows = down.shape[0]
+    _gpu(down, "down", attn.dtype)
+    _gpu(out, "out", attn.dtype)
+    in_dim = attn.numel() // max(1, rows * n_heads)
+    if not (attn.is_contiguous() and attn.numel() == rows * n_heads * in_dim and in_dim >= v_dim):
+        raise KernelError("head_gate: attn must be contiguous [rows, heads, >= v_dim]")
+    if not (out.shape == (rows, n_heads * v_dim) and out.is_contiguous()):
+        raise KernelError("head_gate: out must be contiguous [rows, heads * v_dim]")
+    if not (down.stride(1) == 1 and 0 <= g_col and g_col + n_heads <= down.shape[1]):
+        raise KernelError("head_gate: the gates lie outside down's columns")
+    _check(_fn("latent", "dryft_head_gate")(_ptr(attn), _ptr(down), down.stride(0), g_col, _ptr(out), rows, n_heads,
+                                            in_dim, v_dim, _float_flag(attn, "attn"), _stream()), "head_gate")
+
+
+# ------------------------------------------------------------------------------------------ routed experts
+MOE_MAX_EXPERTS = 512
+MOE_TILE = 32
+
+
+def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale: float, chosen, weights) -> None:
+    """Per row of float32 ``logits`` (their first ``n_experts`` columns): the ``top`` experts by ``sigmoid + correction``
+    among the ``keep`` best of ``groups`` groups (a group's score: its two largest such scores), and their weights
+    ``sigmoid / (sum of the chosen sigmoids + 1e-20) * scale``. ``chosen`` int32 and ``weights`` float32 ``[rows, top]``."""
+    _gpu(logits, "logits", torch.float32)
+    rows, top = chosen.shape
+    if not (logits.dim() == 2 and logits.shape[0] == rows and logits.stride(1) == 1 and logits.shape[1] >= n_experts):
+        raise KernelError("moe_route: logits must be float32 [rows, >= experts] with unit column stride")
+    _f32_vector(correction, "correction", n_experts)
+    _gpu(chosen, "chosen", torch.int32)
+    _gpu(weights, "weights", torch.float32)
+    if not (chosen.is_contiguous() and weights.shape == (rows, top) and weights.is_contiguous()):
+        raise KernelError("moe_route: chosen and weights must be contiguous [rows, top]")
+    if not (1 <= top <= n_experts <= MOE_MAX_EXPERTS and 1 <= keep <= groups <= 64 and n_experts % groups == 0 and
+            keep * (n_experts // groups) >= top):
+        raise KernelError("moe_route: sizes the router does not take")
+    _check(_fn("moe", "dryft_moe_route")(_ptr(logits), logits.stride(0), _ptr(correction), n_experts, groups, keep, top,
+                                         float(scale), _ptr(chosen), _ptr(weights), rows, _stream()), "moe_route")
+
+
+class MoePlan:
+    """Where each (row, expert) pair of a step sits once the pairs are sorted by expert, and the tiles of the sorted
+    run, all on the device."""
+
+    def __init__(self, n_pairs: int, n_experts: int, device):
+        self.n_pairs = n_pairs
+        self.max_tiles = n_pairs // MOE_TILE + min(n_experts, n_pairs)
+        i32 = dict(dtype=torch.int32, device=device)
+        self.sorted_pair = torch.empty(n_pairs, **i32)
+        self.place_of = torch.empty(n_pairs, **i32)
+        self.tiles = torch.empty((3, self.max_tiles), **i32)        # expert | first place | places
+        self.n_tiles = torch.empty(1, **i32)
+
+
+def moe_plan(chosen, n_experts: int) -> MoePlan:
+    _gpu(chosen, "chosen", torch.int32)
+    if not chosen.is_contiguous():
+        raise KernelError("moe_plan: chosen must be contiguous")
+    plan = MoePlan(chosen.numel(), n_experts, chosen.device)
+    _check(_fn("moe", "dryft_moe_plan")(_ptr(chosen), plan.n_pairs, n_experts, _ptr(plan.sorted_pair), _ptr(plan.place_of),
+                                        _ptr(plan.tiles[0]), _ptr(plan.tiles[1]), _ptr(plan.tiles[2]), _ptr(plan.n_tiles),
+                                        plan.max_tiles, _stream()), "moe_plan")
+    return plan
+
+
+def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple[float, float] | None = None) -> None:
+    """``out[place] = W_e a_row`` for every place of the plan, ``e`` the place's expert. ``top`` > 0: ``a`` is
+    ``[rows, K]`` and a place's operand is row ``pair // top``; ``top`` == 0: ``a`` is ``[pairs, K]`` in place order.
+    ``w`` is ``[experts, N, K]``; with ``glu = (limit, alpha)`` it holds gate rows then up rows (``N = 2 I``) and
+    ``out [pairs, I]`` receives the clamped gated unit of the two. ``out`` may be float32 for a plain product."""
+    _gpu(a, "a")
+    _gpu(w, "w", a.dtype)
+    _gpu(out, "out")
+    k = a.shape[1]
+    n_out = w.shape[1] // 2 if glu else w.shape[1]
+    if not (a.dim() == 2 and a.stride(1) == 1 and w.dim() == 3 and w.shape[2] == k and w.is_contiguous()):
+        raise KernelError("moe_products: a [rows, K] with unit column stride, w contiguous [experts, N, K]")
+    if top == 0 and a.shape[0] != plan.n_pairs:
+        raise KernelError("moe_products: an operand in place order needs a row per pair")
+    if top > 0 and a.shape[0] * top != plan.n_pairs:
+        raise KernelError("moe_products: the plan was made for another number of rows")
+    if not (out.shape == (plan.n_pairs, n_out) and out.is_contiguous() and out.dtype in (a.dtype, torch.float32)):
+        raise KernelError(f"moe_products: out must be contiguous [{plan.n_pairs}, {n_out}] in a's dtype or float32")
+    if glu and out.dtype != a.dtype:
+        raise KernelError("moe_products: the gated unit is stored in the activation dtype")
+    limit, alpha = glu if glu else (0.0, 0.0)
+    _check(_fn("moe", "dryft_moe_product")(
+        _ptr(a), a.stride(0), _ptr(w), _ptr(plan.sorted_pair), _ptr(plan.tiles[0]), _ptr(plan.tiles[1]),
+        _ptr(plan.tiles[2]), _ptr(plan.n_tiles), plan.max_tiles, _ptr(out), 1 if out.dtype == torch.float32 else 0,
+        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), _float_flag(a, "a"), _stream()), "moe_products")
+
+
+def moe_combine(y, plan: MoePlan, weights, shared, logits, shared_col: int, out) -> None:
+    """``out[row] = sum_k weights[row, k] * y[place of (row, k)] + sigmoid(logits[row, shared_col]) * shared[row]``
+    (the last term only with ``shared``)."""
+    _gpu(y, "y", torch.float32)
+    rows, top = weights.shape
+    width = y.shape[1]
+    _gpu(weights, "weights", torch.float32)
+    _gpu(out, "out")
+    if not (y.shape == (rows * top, width) and y.is_contiguous() and weights.is_contiguous() and
+            out.shape == (rows, width) and out.is_contiguous() and plan.n_pairs == rows * top):
+        raise KernelError("moe_combine: y [pairs, width], weights [rows, top], out [rows, width], all contiguous")
+    if shared is not None:
+        _gpu(shared, "shared", out.dtype)
+        _gpu(logits, "logits", torch.float32)
+        if not (shared.shape == (rows, width) and shared.is_contiguous() and logits.stride(1) == 1 and
+                0 <= shared_col < logits.shape[1] and logits.shape[0] == rows):
+            raise KernelError("moe_combine: shared [rows, width] contiguous, its logit a column of logits")
+    _check(_fn("moe", "dryft_moe_combine")(_ptr(y), _ptr(plan.place_of), _ptr(weights), _ptr(shared), _ptr(logits),
+                                           logits.stride(0) if shared is not None else 0, shared_col, _ptr(out), rows, top,
+                                           width, _float_flag(out, "out"), _stream()), "moe_combine")

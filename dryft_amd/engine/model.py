@@ -192,5 +192,8 @@ def _pick_rows(x, rows: torch.Tensor):
         parts = x.data[:x.count]
         picked = torch.empty((x.count, rows.numel(), parts.shape[2]), dtype=parts.dtype, device=parts.device)
         return Partials(ops.embed_rows(rows, parts, picked), x.count)
+    if x.dim() == 3:                                            # a stream of several copies: the rows of each
+        picked = torch.empty((x.shape[0], rows.numel(), x.shape[2]), dtype=x.dtype, device=x.device)
+        return ops.embed_rows(rows, x, picked)
     picked = torch.empty((rows.numel(), x.shape[1]), dtype=x.dtype, device=x.device)
     return ops.embed_rows(rows, x, picked)

@@ -120,16 +120,18 @@ class Deferred:
     """What has still to be added to a float32 residual stream before the next norm reads it, so that one kernel
     can do all of it: a branch's output ``delta`` (a tensor or ``Partials``) that is normed with ``norm`` first (None:
     added as it is), a tensor ``rows`` in the activation dtype that is added row by row (the embedding's output coming
-    back), and a ``vector`` added to every row."""
+    back), and a ``vector`` added to every row. On a stream of several copies, ``route`` says how ``delta`` enters:
+    the part that holds the weights with which the copies are mixed and with which each takes the output."""
 
     delta: Any = None
     norm: Any = None
     rows: torch.Tensor | None = None
     vector: torch.Tensor | None = None
+    route: Any = None
 
     def picked(self, pick) -> "Deferred":
         """The same for a choice of rows; ``pick`` gathers them from a tensor or from partial sums."""
-        return Deferred(pick(self.delta), self.norm, pick(self.rows), self.vector)
+        return Deferred(pick(self.delta), self.norm, pick(self.rows), self.vector, self.route)
 
 
 class Part:

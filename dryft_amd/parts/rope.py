@@ -85,5 +85,29 @@ class PairRotaryPositions(PositionEncoding):
         self.n_positions = n_positions
 
 
+class HalfRotaryPositions(PositionEncoding):
+    """Float32 tables for a rotation that pairs feature ``i`` with feature ``i + dims/2`` of the first ``dims``
+    features of a vector: ``cos``/``sin`` are ``[positions, dims / 2]`` of the angles ``p * base^(-2i / dims)``, formed
+    in float64 on the host and rounded once, whatever the activation dtype."""
+
+    def __init__(self, dims: int, base: float):
+        if dims % 2 or dims <= 0:
+            raise ValueError(f"the rotated width must be even and positive, got {dims}")
+        self.dims, self.base = int(dims), float(base)
+        self.cos: torch.Tensor | None = None
+        self.sin: torch.Tensor | None = None
+        self.n_positions = 0
+
+    def prepare(self, n_positions: int, dtype: torch.dtype, device) -> None:
+        if self.cos is not None and n_positions <= self.n_positions:
+            return
+        f = self.base ** (-2.0 * torch.arange(self.dims // 2, dtype=torch.float64) / self.dims)
+        angle = torch.arange(n_positions, dtype=torch.float64)[:, None] * f[None, :]
+        self.cos = angle.cos().to(torch.float32).to(device).contiguous()
+        self.sin = angle.sin().to(torch.float32).to(device).contiguous()
+        self.n_positions = n_positions
+
+
 register_part("rotary", RotaryPositions)
+register_part("half_rotary", HalfRotaryPositions)
 register_part("pair_rotary", PairRotaryPositions)

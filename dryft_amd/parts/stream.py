@@ -24,20 +24,26 @@ from .base import Deferred, FeedForward, Mixer, Norm, Partials, StepContext, Str
 
 
 class StreamRMSNorm(Norm):
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = int(size), float(eps)
+    """``offset``: what the stored weight is counted from (1 for weights stored around zero); ``scale``: a factor on
+    the whole weight (a head's factor on its logits rides here). A stream of several copies ``[copies, rows, width]``
+    (``parts/hyper.py``) is normed as the sum of its copies."""
+
+    def __init__(self, size: int, eps: float, offset: float = 0.0, scale: float = 1.0):
+        self.size, self.eps, self.offset, self.scale = int(size), float(eps), float(offset), float(scale)
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self):
-        return {"weight": ((self.size,), VECTOR, "ones")}
+        return {"weight": ((self.size,), VECTOR, "zeros" if self.offset == 1.0 else "ones")}
 
     def load(self, tensors):
-        self.weight = tensors["weight"].float()
+        self.weight = ((tensors["weight"].float() + self.offset) * self.scale).contiguous()
 
     def kernel_modules(self, dtype):
         return ("norm",)
 
     def forward(self, x: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+        if x.dim() == 3:
+            return self.add_forward(x, None, dtype)[1]
         y = torch.empty(x.shape, dtype=dtype or self.compute_dtype or x.dtype, device=x.device)
         ops.stream_norm(x, None, None, None, None, self.weight, self.eps, None, y, y.dtype)
         return y
@@ -48,6 +54,9 @@ class StreamRMSNorm(Norm):
         ``in_place`` allows; the normed rows in ``dtype`` (default: the dtype the model computes in)."""
         pending = as_deferred(delta)
         act = dtype or self.compute_dtype or _activation_dtype(res, pending)
+        if res.dim() == 3 or pending.route is not None:
+            from .hyper import read_streams
+            return read_streams(res, pending, None, self, act, keep=False)
         own = in_place and res.dtype == torch.float32 and res.is_contiguous()
         out = res if own else torch.empty(res.shape, dtype=torch.float32, device=res.device)
         y = torch.empty(res.shape, dtype=act, device=res.device)
@@ -84,6 +93,9 @@ def settle(x: torch.Tensor, pending, eps: float = 0.0) -> torch.Tensor:
     """The stream with everything pending added, as a new float32 tensor (for looking at it; the compute path never
     needs the stream without the norm that follows)."""
     pending = as_deferred(pending)
+    if x.dim() == 3 or pending.route is not None:
+        from .hyper import summed_streams
+        return summed_streams(x, pending)
     out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
     act = _activation_dtype(x, pending)
     _launch(x, pending, None, pending.norm.eps if pending.norm is not None else eps, out, None, act)

@@ -111,6 +111,12 @@ def stored_dtype_to_held(stored: torch.dtype, role: str, compute_dtype: torch.dt
     return torch.bfloat16
 
 
+def shape_fits(stored: tuple[int, ...], wanted: tuple[int, ...]) -> bool:
+    """Does a stored shape fit a spec's? An extent of -1 in the spec is free: the file decides it (a rank that no
+    configuration key gives), and the part that reads the tensor checks it against its other tensors."""
+    return len(stored) == len(wanted) and all(w == -1 or w == g for g, w in zip(stored, wanted))
+
+
 def load_tensors(model_dir: str, specs: Iterable[TensorSpec], compute_dtype: torch.dtype,
                  device: torch.device | str = "cpu", ignore: Iterable[str] = ()) -> dict[str, torch.Tensor]:
     """All tensors named by ``specs`` from the checkpoint in ``model_dir``.
@@ -132,7 +138,7 @@ def load_tensors(model_dir: str, specs: Iterable[TensorSpec], compute_dtype: tor
                 got = shards.shape(s.name)
                 if got is None:                       # the index names a shard that does not hold it
                     missing.append(s.name)
-                elif got != tuple(s.shape):
+                elif not shape_fits(got, s.shape):
                     wrong.append((s.name, tuple(s.shape), got))
         if missing or unexpected or wrong:
             raise WeightError(model_dir, missing, unexpected, wrong)

@@ -32,8 +32,14 @@ def random_tensors(specs: Iterable[TensorSpec], seed: int, dtype: torch.dtype = 
     for s in specs:
         if s.role == INT_TABLE:
             raise ValueError(f"{s.name}: integer tables have no random initialiser")
-        if s.init == "ones":
-            t = torch.ones(s.shape, dtype=torch.float32, device=device)
+        if any(d < 0 for d in s.shape):
+            raise ValueError(f"{s.name}: an extent that only a checkpoint decides has no random initialiser; "
+                             "give it in the configuration")
+        if s.init in ("ones", "zeros", "eye"):
+            if s.init == "eye":
+                t = torch.eye(s.shape[0], s.shape[1], dtype=torch.float32, device=device)
+            else:
+                t = torch.full(s.shape, 1.0 if s.init == "ones" else 0.0, dtype=torch.float32, device=device)
             if norm_std:
                 t += norm_std * torch.randn(s.shape, generator=gen, dtype=torch.float32, device=device)
         else:

@@ -14,10 +14,10 @@ class TensorSpec:
     name: str                      # name in the checkpoint
     shape: tuple[int, ...]
     role: str = MATRIX
-    init: str = "normal"           # random-weights mode: "normal" or "ones"
+    init: str = "normal"           # random-weights mode: "normal", "ones", "zeros" or "eye" (a unit matrix)
 
     def __post_init__(self):
         if self.role not in (MATRIX, VECTOR, INT_TABLE):
             raise ValueError(f"{self.name}: unknown role {self.role!r}")
-        if self.init not in ("normal", "ones"):
+        if self.init not in ("normal", "ones", "zeros", "eye"):
             raise ValueError(f"{self.name}: unknown init {self.init!r}")
