@@ -1305,12 +1305,14 @@ def rglru_scan_tiles(coef, proj, x_col: int, y_col: int, x_bias, y_bias, taps: i
 HYPER_MAX_STREAMS = 8
 
 
-def hyper_norm(x, n: int, delta, mix, write, read, weight, eps: float, x_out, y, *, normed: bool) -> None:
+def hyper_norm(x, n: int, delta, mix, write, read, weight, eps: float, x_out, y, *, normed: bool, act=None) -> None:
     """One launch for a residual stream of ``n`` copies: ``x'_t = sum_s mix[s, t] x_s + write[t] * delta`` (skipped
     without ``delta``), written to ``x_out [n, rows, width]`` (float32, may be ``x``; None: not kept);
     ``u = sum_t read[t] x'_t`` (``read`` None: the plain sum); ``y = rmsnorm(u) * weight`` in the activation dtype
     when ``normed``, else ``y = u`` in float32. ``x`` is the copies in float32 or one ``[rows, width]`` tensor in the
-    activation dtype that every copy equals; ``delta`` a tensor in the activation dtype or ``(partials, count)``."""
+    activation dtype that every copy equals; ``delta`` a tensor in the activation dtype or ``(partials, count)``
+    (partial sums are rounded to the activation dtype once added up, as the product itself would have stored them;
+    ``act`` names that dtype where no operand shows it)."""
     _gpu(x, "x")
     rows, width = x.shape[-2:]
     copies = x.dim() == 3
@@ -1321,7 +1323,8 @@ def hyper_norm(x, n: int, delta, mix, write, read, weight, eps: float, x_out, y,
         raise KernelError("hyper_norm: a stream that starts must be contiguous [rows, width]")
     if not 1 <= n <= HYPER_MAX_STREAMS:
         raise KernelError(f"hyper_norm: 1..{HYPER_MAX_STREAMS} copies, got {n}")
-    act = y.dtype if (y is not None and normed) else (x.dtype if not copies else None)
+    if act is None:
+        act = y.dtype if (y is not None and normed) else (x.dtype if not copies else None)
     kind, n_partials, stride = 0, 0, 0
     if delta is not None:
         data, n_partials = delta if isinstance(delta, tuple) else (delta, 1)

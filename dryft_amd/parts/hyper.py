@@ -85,7 +85,7 @@ def summed_streams(x: torch.Tensor, pending: Deferred) -> torch.Tensor:
         delta = (delta.data, delta.count)
     taken = pending.route
     ops.hyper_norm(x, n, delta, taken.mix if taken else None, taken.write if taken else None, None, None, 0.0, None,
-                   out, normed=False)
+                   out, normed=False, act=taken.compute_dtype if taken else None)
     return out
 
 
