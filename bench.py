@@ -128,12 +128,42 @@ def compare_designs(args) -> int:
     return 0
 
 
+def compare_fetedra(args) -> int:
+    """``--design fetedra``: Fetedra at a few sizes with the widths of real models' layers beside the Piralix preset of
+    the same width (the closest design the library has: mixed recurrent and attention layers on a float32 stream;
+    the presets of a width hold about the same weight bytes); random weights, bfloat16, one prompt of
+    ``--prompt-len`` tokens and ``--batch`` sequences decoding. One JSON line."""
+    import torch
+
+    from dryft_amd import Engine
+    from dryft_amd.models import load_preset
+
+    sizes = []
+    for name in args.sizes.split(","):
+        raw = load_preset(name)
+        kw = dict(seed=args.seed, dtype="bfloat16", max_batch=args.batch, max_len=args.prompt_len + 2 * (args.steps + args.warmup) + 64,
+                  use_graph=not args.no_graph)
+        entry = {"preset": name, "width": raw["width"], "layers": len(raw["layers"])}
+        for key, cfg in (("fetedra", raw), ("piralix", load_preset(f"piralix-w{raw['width']}"))):
+            engine = Engine(config=cfg, **kw)
+            entry[key] = measure(engine, args.prompt_len, args.batch, args.steps, args.warmup, args.seed)
+            del engine
+            torch.cuda.empty_cache()
+        sizes.append(entry)
+    print(json.dumps({"metric": "prefill and decode of Fetedra beside Piralix of equal width",
+                      "dtype": "bf16", "data": "synthetic (random weights, uniform random token ids)",
+                      "prompt_len": args.prompt_len, "batch": args.batch, "steps": args.steps, "warmup": args.warmup,
+                      "graph": not args.no_graph, "sizes": sizes}))
+    return 0
+
+
 def main() -> int:
     global PROMPT, SLOT
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["piralix"],
-                    help="instead of the default workload: that design beside Qwen3 at equal size (one JSON line)")
-    ap.add_argument("--sizes", default="piralix-w1024,piralix-w2048,piralix-w2560", help="presets for --design")
+    ap.add_argument("--design", default=None, choices=["piralix", "fetedra"],
+                    help="instead of the default workload: that design beside its closest relative in the library at "
+                         "equal size (Piralix beside Qwen3, Fetedra beside Piralix; one JSON line)")
+    ap.add_argument("--sizes", default=None, help="presets for --design (default: the design's presets)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
@@ -154,7 +184,9 @@ def main() -> int:
     PROMPT = args.prompt_len
     SLOT = args.slot_len or max(SLOT, 2 * PROMPT)
     if args.design:
-        return compare_designs(args)
+        args.sizes = args.sizes or {"piralix": "piralix-w1024,piralix-w2048,piralix-w2560",
+                                    "fetedra": "fetedra-w1024,fetedra-w2048"}[args.design]
+        return compare_fetedra(args) if args.design == "fetedra" else compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")
         return 2

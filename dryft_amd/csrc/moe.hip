@@ -5,7 +5,7 @@
 
 #define MOE_MAX_EXPERTS 512
 #define MOE_PER_LANE (MOE_MAX_EXPERTS / WAVE)
-#define MOE_TILE 32            // pairs of one expert that a workgroup of the products takes
+#define MOE_TILE 64            // pairs of one expert that a workgroup of the products takes
 
 struct Best {
   float v;
@@ -171,7 +171,7 @@ DRYFT_API int dryft_moe_plan(const int* chosen, int n_pairs, int n_experts, int*
 
 // ---------------------------------------------------------------------------------------------------
 // Grouped product, plain multiply-adds: for every tile of an expert's places, out[place] = W_e a[place]. A
-// workgroup takes one tile (up to 32 places) and 64 outputs; K goes through LDS 32 at a time; a thread owns two
+// workgroup takes one tile (up to 64 places) and 64 outputs; K goes through LDS 32 at a time; a thread owns four
 // places and four outputs. With `top` > 0 the operand rows are gathered: place -> pair -> row pair / top of `a`;
 // otherwise `a` is already in place order. GLU: W_e holds gate rows then up rows; the clamped gated unit
 // g * sigmoid(alpha g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit), is applied to the float
@@ -198,10 +198,11 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
   const T* we = w + (int64_t)expert * w_rows * k_dim;
   if (threadIdx.x < MOE_TILE)
     src_row[threadIdx.x] = threadIdx.x < count ? (top > 0 ? sorted_pair[start + threadIdx.x] / top : start + threadIdx.x) : -1;
-  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;      // places ty, ty + 16; outputs tx + 16 j
-  float acc[2][4], acc_up[2][4];
+  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;      // places ty + 16 i; outputs tx + 16 j
+  constexpr int PM = MOE_TILE / 16;
+  float acc[PM][4], acc_up[PM][4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < PM; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = acc_up[i][j] = 0.f;
   for (int k0 = 0; k0 < k_dim; k0 += MOE_TK) {
@@ -220,22 +221,23 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
     __syncthreads();
 #pragma unroll 8
     for (int kk = 0; kk < MOE_TK; ++kk) {
-      const float a0 = sa[ty][kk], a1 = sa[ty + 16][kk];
+      float av[PM];
+#pragma unroll
+      for (int i = 0; i < PM; ++i) av[i] = sa[ty + 16 * i][kk];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float b = sw[tx + 16 * j][kk];
-        acc[0][j] += a0 * b;
-        acc[1][j] += a1 * b;
-        if (GLU) {
-          const float u = sw[MOE_TN + tx + 16 * j][kk];
-          acc_up[0][j] += a0 * u;
-          acc_up[1][j] += a1 * u;
+        const float u = GLU ? sw[MOE_TN + tx + 16 * j][kk] : 0.f;
+#pragma unroll
+        for (int i = 0; i < PM; ++i) {
+          acc[i][j] += av[i] * b;
+          if (GLU) acc_up[i][j] += av[i] * u;
         }
       }
     }
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < PM; ++i) {
     const int r = ty + 16 * i;
     if (r >= count) continue;
 #pragma unroll
@@ -254,6 +256,79 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
   }
 }
 
+// The same on the matrix cores (bfloat16, K a multiple of 8, rows at 16-byte addresses). A wave owns 16 outputs (for
+// the gated unit 16 gate rows and the 16 up rows that go with them) and all 64 places of the tile: the weights are the
+// first operand of v_mfma_f32_16x16x32_bf16 (lane c + 16 g holds row c, values 8 g .. 8 g + 7 of a block of 32), the
+// operand rows the second, so accumulator entry i of lane (c, g) is output 4 g + i of place c. Operands go straight
+// from memory into that layout, 16 bytes a lane; every weight is read by one wave of the workgroup.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <typename O, bool GLU>
+__global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __restrict__ a, int64_t a_stride,
+                                                               const bf16_t* __restrict__ w,
+                                                               const int* __restrict__ sorted_pair,
+                                                               const int* __restrict__ tile_expert,
+                                                               const int* __restrict__ tile_start,
+                                                               const int* __restrict__ tile_rows,
+                                                               const int* __restrict__ n_tiles, O* __restrict__ out,
+                                                               int top, int n_out, int k_dim, float limit, float alpha) {
+  constexpr int MT = MOE_TILE / 16;
+  const int tile = blockIdx.x;
+  if (tile >= *n_tiles) return;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  if (n0 >= n_out) return;
+  const int expert = tile_expert[tile], start = tile_start[tile], count = tile_rows[tile];
+  const int w_rows = GLU ? 2 * n_out : n_out;
+  const bf16_t* we = w + (int64_t)expert * w_rows * k_dim;
+  const int n_mine = min(n0 + c, n_out - 1);                  // rows beyond the last are read from it and never stored
+  const bf16_t* w_gate = we + (int64_t)n_mine * k_dim + 8 * g;
+  const bf16_t* w_up = we + ((int64_t)n_out + n_mine) * k_dim + 8 * g;
+  const bf16_t* rows[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int place = start + min(16 * mt + c, count - 1);    // places beyond the tile's: its last one, never stored
+    const int row = top > 0 ? sorted_pair[place] / top : place;
+    rows[mt] = a + (int64_t)row * a_stride + 8 * g;
+  }
+  f32x4 acc[MT], acc_up[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_up[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int k0 = 0; k0 < k_dim; k0 += 32) {
+    const bool in = k0 + 8 * g < k_dim;                       // K is a multiple of 8: a lane's eight are in or out
+    const bf16x8 wg = in ? *(const bf16x8*)(w_gate + k0) : zero;
+    bf16x8 wu = zero;
+    if (GLU && in) wu = *(const bf16x8*)(w_up + k0);
+    bf16x8 x[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) x[mt] = in ? *(const bf16x8*)(rows[mt] + k0) : zero;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg, x[mt], acc[mt], 0, 0, 0);
+      if (GLU) acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu, x[mt], acc_up[mt], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = 16 * mt + c;
+    if (m >= count) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= n_out) continue;
+      float v = acc[mt][i];
+      if (GLU) {
+        const float gv = fminf(rounded_as<bf16_t>(v), limit);
+        const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[mt][i]), -limit), limit);
+        v = gv / (1.f + expf(-alpha * gv)) * (uv + 1.f);
+      }
+      store_from_float(out + (int64_t)(start + m) * n_out + n, v);
+    }
+  }
+}
+
 DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, const int* sorted_pair,
                                 const int* tile_expert, const int* tile_start, const int* tile_rows, const int* n_tiles,
                                 int max_tiles, void* out, int out_is_f32, int top, int n_out, int k_dim, int glu,
@@ -261,6 +336,17 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || k_dim <= 0 || (glu && out_is_f32 && !is_f32)) return -1;
   dim3 grid(max_tiles, (n_out + MOE_TN - 1) / MOE_TN), block(256);
+  if (!is_f32 && k_dim % 8 == 0 && a_stride % 8 == 0 && (((uintptr_t)a | (uintptr_t)w) & 15) == 0) {
+#define MOE_MFMA(O, G)                                                                                            \
+  hipLaunchKernelGGL((moe_product_mfma_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,          \
+                     (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
+                     k_dim, limit, alpha)
+    if (glu) MOE_MFMA(bf16_t, true);
+    else if (out_is_f32) MOE_MFMA(float, false);
+    else MOE_MFMA(bf16_t, false);
+#undef MOE_MFMA
+    return DRYFT_LAUNCH_CHECK();
+  }
 #define MOE_LAUNCH(T, O, G)                                                                                       \
   hipLaunchKernelGGL((moe_product_kernel<T, O, G>), grid, block, 0, stream, (const T*)a, a_stride, (const T*)w,   \
                      sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha)

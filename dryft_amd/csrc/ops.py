@@ -1540,7 +1540,7 @@ def head_gate(attn, down, g_col: int, out, n_heads: int, v_dim: int) -> None:
 
 # ------------------------------------------------------------------------------------------ routed experts
 MOE_MAX_EXPERTS = 512
-MOE_TILE = 32
+MOE_TILE = 64
 
 
 def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale: float, chosen, weights) -> None:

@@ -101,44 +101,49 @@ DRYFT_API int dryft_wkv_decay(const float* low, const void* up, const float* bia
 }
 
 // ---------------------------------------------------------------------------------------------------
-// The recurrence, token by token. One wave per (sequence, head, run of 64 value columns); lane j keeps column j of
-// the state S [dim, dim] in registers. Per token, with r, k, w = exp(log w) and the bonus u shared through LDS:
+// The recurrence, token by token. A wave takes 16 value columns of one (sequence, head): lane (c, q) keeps a quarter
+// of column c of the state S [dim, dim] in registers (key channels q DK/4 .. (q+1) DK/4 - 1). The waves of a
+// workgroup (up to four: 64 columns) share r, k, w = exp(log w) and the bonus u of eight tokens at a time through
+// LDS. Per token
 //
 //   o_j = sum_i r_i S_ij + v_j sum_i r_i u_i k_i ;   S_ij <- w_i S_ij + k_i v_j
 //
-// Tokens come to LDS eight at a time. The wave of head 0 and column run 0 also keeps the sequence's last input row
-// as the next step's h' (`previous`), after every row of the step has been blended by the launch before.
+// with the sums over a lane's quarter first and over the four quarters by two exchanges between lanes. The wave of
+// head 0 and column 0 also keeps the sequence's last input row as the next step's h' (`previous`), after every row
+// of the step has been blended by the launch before.
 #define WKV_GROUP 8
 
 template <typename T, int DK>
-__global__ __launch_bounds__(64) void wkv_steps_kernel(const T* __restrict__ r, const T* __restrict__ k,
-                                                       const T* __restrict__ v, const float* __restrict__ log_w,
-                                                       const float* __restrict__ bonus, const int* __restrict__ seq_slot,
-                                                       const int* __restrict__ cu_rows, const int* __restrict__ q_len,
-                                                       float* __restrict__ state, float* __restrict__ o_raw,
-                                                       const T* __restrict__ h, float* __restrict__ previous, int hidden,
-                                                       int n_heads, int dim, int write_state) {
-  __shared__ float sh_r[WKV_GROUP][DK], sh_k[WKV_GROUP][DK], sh_w[WKV_GROUP][DK], sh_u[DK];
-  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * WAVE + lane;
+__global__ __launch_bounds__(256) void wkv_steps_kernel(const T* __restrict__ r, const T* __restrict__ k,
+                                                        const T* __restrict__ v, const float* __restrict__ log_w,
+                                                        const float* __restrict__ bonus, const int* __restrict__ seq_slot,
+                                                        const int* __restrict__ cu_rows, const int* __restrict__ q_len,
+                                                        float* __restrict__ state, float* __restrict__ o_raw,
+                                                        const T* __restrict__ h, float* __restrict__ previous, int hidden,
+                                                        int n_heads, int dim, int write_state) {
+  constexpr int DQ = DK / 4;
+  __shared__ __attribute__((aligned(16))) float sh_r[WKV_GROUP][DK], sh_k[WKV_GROUP][DK], sh_w[WKV_GROUP][DK], sh_u[DK];
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, q = lane / 16;
+  const int col = (blockIdx.z * (blockDim.x / WAVE) + wave) * 16 + c;
   const int slot = seq_slot[seq], row0 = cu_rows[seq], n = q_len[seq];
   const int inner = n_heads * dim;
   const bool owns = col < dim;
   if (slot < 0) {                      // a sequence that sits out: its rows of the output hold zeros
     for (int t = 0; t < n; ++t)
-      if (owns) o_raw[(int64_t)(row0 + t) * inner + head * dim + col] = 0.f;
+      if (owns && q == 0) o_raw[(int64_t)(row0 + t) * inner + head * dim + col] = 0.f;
     return;
   }
   if (n <= 0) return;
-  float S[DK];
-  float* s_col = state + (((int64_t)slot * n_heads + head) * dim) * dim + col;
+  float S[DQ];
+  float* s_col = state + (((int64_t)slot * n_heads + head) * dim + q * DQ) * dim + col;
 #pragma unroll
-  for (int i = 0; i < DK; ++i) S[i] = (owns && i < dim) ? s_col[(int64_t)i * dim] : 0.f;
-  for (int i = lane; i < DK; i += WAVE) sh_u[i] = i < dim ? bonus[head * dim + i] : 0.f;
+  for (int i = 0; i < DQ; ++i) S[i] = (owns && q * DQ + i < dim) ? s_col[(int64_t)i * dim] : 0.f;
+  for (int i = threadIdx.x; i < DK; i += blockDim.x) sh_u[i] = i < dim ? bonus[head * dim + i] : 0.f;
   for (int t0 = 0; t0 < n; t0 += WKV_GROUP) {
     const int g = min(WKV_GROUP, n - t0);
     __syncthreads();
-    for (int e = lane; e < g * DK; e += WAVE) {
+    for (int e = threadIdx.x; e < g * DK; e += blockDim.x) {
       const int t = e / DK, i = e % DK;
       const int64_t at = (int64_t)(row0 + t0 + t) * inner + head * dim + i;
       const bool in = i < dim;
@@ -146,28 +151,39 @@ __global__ __launch_bounds__(64) void wkv_steps_kernel(const T* __restrict__ r, 
       sh_k[t][i] = in ? load_as_float(k + at) : 0.f;
       sh_w[t][i] = in ? expf(log_w[at]) : 0.f;
     }
+    float vj[WKV_GROUP];
+#pragma unroll
+    for (int t = 0; t < WKV_GROUP; ++t)
+      vj[t] = (owns && t < g) ? load_as_float(v + (int64_t)(row0 + t0 + t) * inner + head * dim + col) : 0.f;
     __syncthreads();
-    for (int t = 0; t < g; ++t) {
-      const int64_t at = (int64_t)(row0 + t0 + t) * inner + head * dim + col;
-      const float vj = owns ? load_as_float(v + at) : 0.f;
+#pragma unroll
+    for (int t = 0; t < WKV_GROUP; ++t) {
+      if (t >= g) break;
       float o = 0.f, ruk = 0.f;
 #pragma unroll
-      for (int i = 0; i < DK; ++i) {
-        const float ri = sh_r[t][i], ki = sh_k[t][i];
-        o += ri * S[i];
-        ruk += ri * sh_u[i] * ki;
-        S[i] = sh_w[t][i] * S[i] + ki * vj;
+      for (int i = 0; i < DQ; i += 4) {
+        const vf4 r4 = *(const vf4*)&sh_r[t][q * DQ + i], k4 = *(const vf4*)&sh_k[t][q * DQ + i];
+        const vf4 w4 = *(const vf4*)&sh_w[t][q * DQ + i], u4 = *(const vf4*)&sh_u[q * DQ + i];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o += r4[e] * S[i + e];
+          ruk += r4[e] * u4[e] * k4[e];
+          S[i + e] = w4[e] * S[i + e] + k4[e] * vj[t];
+        }
       }
-      if (owns) o_raw[at] = o + vj * ruk;
+      o += vj[t] * ruk;
+      o += __shfl_xor(o, 16, WAVE);
+      o += __shfl_xor(o, 32, WAVE);
+      if (owns && q == 0) o_raw[(int64_t)(row0 + t0 + t) * inner + head * dim + col] = o;
     }
   }
   if (!write_state) return;
 #pragma unroll
-  for (int i = 0; i < DK; ++i)
-    if (owns && i < dim) s_col[(int64_t)i * dim] = S[i];
-  if (head == 0 && blockIdx.z == 0) {
+  for (int i = 0; i < DQ; ++i)
+    if (owns && q * DQ + i < dim) s_col[(int64_t)i * dim] = S[i];
+  if (head == 0 && blockIdx.z == 0 && wave == 0) {
     const T* last = h + (int64_t)(row0 + n - 1) * hidden;
-    for (int c = lane; c < hidden; c += WAVE) previous[(int64_t)slot * hidden + c] = load_as_float(last + c);
+    for (int cc = lane; cc < hidden; cc += WAVE) previous[(int64_t)slot * hidden + cc] = load_as_float(last + cc);
   }
 }
 
@@ -176,7 +192,8 @@ static int launch_wkv_steps(hipStream_t stream, const void* r, const void* k, co
                             const float* bonus, const int* seq_slot, const int* cu_rows, const int* q_len, int n_seqs,
                             float* state, float* o_raw, const void* h, float* previous, int hidden, int n_heads, int dim,
                             int write_state) {
-  dim3 grid(n_seqs, n_heads, (dim + WAVE - 1) / WAVE), block(WAVE);
+  const int waves = min(4, (dim + 15) / 16);                   // 16 value columns a wave
+  dim3 grid(n_seqs, n_heads, (dim + 16 * waves - 1) / (16 * waves)), block(WAVE * waves);
 #define WKV_CASE(DK)                                                                                               \
   hipLaunchKernelGGL((wkv_steps_kernel<T, DK>), grid, block, 0, stream, (const T*)r, (const T*)k, (const T*)v, log_w, \
                      bonus, seq_slot, cu_rows, q_len, state, o_raw, (const T*)h, previous, hidden, n_heads, dim,     \
