@@ -14,7 +14,7 @@
 #define HYPER_MAX 8
 
 template <typename T, int N>
-__global__ __launch_bounds__(256) void hyper_norm_kernel(const void* __restrict__ x_in, int x_is_copies,
+__global__ __launch_bounds__(1024) void hyper_norm_kernel(const void* __restrict__ x_in, int x_is_copies,
                                                          const void* __restrict__ delta, int delta_kind, int n_partials,
                                                          int64_t partial_stride, const float* __restrict__ mix,
                                                          const float* __restrict__ write_w,
@@ -114,7 +114,8 @@ DRYFT_API int dryft_hyper_norm(const void* x, int x_is_copies, int n, const void
   if (n < 1 || n > HYPER_MAX || width <= 0 || width > 16384) return -1;
   if (delta_kind && (mix == nullptr || write_w == nullptr)) return -1;
   if (y && normed && weight == nullptr) return -1;
-  dim3 grid(rows), block(256);
+  // few rows: more threads a row, so that a row's loads are all in flight at once
+  dim3 grid(rows), block(rows <= 128 && width >= 1024 ? 1024 : 256);
   const size_t lds = (size_t)width * sizeof(float);
   if (is_f32)
     return launch_hyper<float>(n, grid, block, lds, stream, x, x_is_copies, delta, delta_kind, n_partials,

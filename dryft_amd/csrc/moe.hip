@@ -28,6 +28,7 @@ __device__ __forceinline__ Best wave_best(Best b) {
 // score is the sum of its two largest choice scores (of its only one, if it has one); experts outside the `keep`
 // best groups drop out. The `top` largest choice scores that remain are chosen, highest first, and weigh
 // s / (sum of the chosen s + 1e-20) * scale. One wave a row; lane l holds experts l, l + 64, ...
+template <int PER>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int64_t stride,
                                                         const float* __restrict__ correction, int n_experts, int groups,
                                                         int keep, int top, float scale, int* __restrict__ chosen,
@@ -36,9 +37,9 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;
   if (row >= rows) return;
   const float NEG = -__builtin_inff();
-  float s[MOE_PER_LANE], c[MOE_PER_LANE];
+  float s[PER], c[PER];
 #pragma unroll
-  for (int j = 0; j < MOE_PER_LANE; ++j) {
+  for (int j = 0; j < PER; ++j) {
     const int e = lane + WAVE * j;
     s[j] = 0.f;
     c[j] = NEG;
@@ -53,7 +54,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     for (int g = 0; g < groups; ++g) {
       Best a{NEG, 0x7fffffff};
 #pragma unroll
-      for (int j = 0; j < MOE_PER_LANE; ++j) {
+      for (int j = 0; j < PER; ++j) {
         const int e = lane + WAVE * j;
         if (e < n_experts && e / size == g && (c[j] > a.v || (c[j] == a.v && e < a.i))) { a.v = c[j]; a.i = e; }
       }
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
       if (size >= 2) {
         Best b{NEG, 0x7fffffff};
 #pragma unroll
-        for (int j = 0; j < MOE_PER_LANE; ++j) {
+        for (int j = 0; j < PER; ++j) {
           const int e = lane + WAVE * j;
           if (e < n_experts && e / size == g && e != a.i && (c[j] > b.v || (c[j] == b.v && e < b.i))) { b.v = c[j]; b.i = e; }
         }
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
       if (a.i < groups) kept |= 1ull << a.i;
     }
 #pragma unroll
-    for (int j = 0; j < MOE_PER_LANE; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int e = lane + WAVE * j;
       if (e < n_experts && !((kept >> (e / size)) & 1)) c[j] = NEG;
     }
@@ -88,14 +89,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   for (int i = 0; i < top; ++i) {
     Best a{NEG, 0x7fffffff};
 #pragma unroll
-    for (int j = 0; j < MOE_PER_LANE; ++j) {
+    for (int j = 0; j < PER; ++j) {
       const int e = lane + WAVE * j;
       if (e < n_experts && (c[j] > a.v || (c[j] == a.v && e < a.i))) { a.v = c[j]; a.i = e; }
     }
     a = wave_best(a);
     float sv = 0.f;
 #pragma unroll
-    for (int j = 0; j < MOE_PER_LANE; ++j)
+    for (int j = 0; j < PER; ++j)
       if (lane + WAVE * j == a.i) { sv = s[j]; c[j] = NEG; }
     sv = wave_sum(sv);
     total += sv;
@@ -117,8 +118,13 @@ DRYFT_API int dryft_moe_route(const float* logits, int64_t stride, const float* 
   if (n_experts < 1 || n_experts > MOE_MAX_EXPERTS || top < 1 || top > n_experts || groups < 1 || groups > WAVE ||
       n_experts % groups || keep < 1 || keep > groups || keep * (n_experts / groups) < top)
     return -1;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, logits, stride, correction, n_experts,
-                     groups, keep, top, scale, chosen, weights, rows);
+#define MOE_ROUTE(PER)                                                                                              \
+  hipLaunchKernelGGL(moe_route_kernel<PER>, dim3((rows + 3) / 4), dim3(256), 0, stream, logits, stride, correction,   \
+                     n_experts, groups, keep, top, scale, chosen, weights, rows)
+  if (n_experts <= WAVE) MOE_ROUTE(1);
+  else if (n_experts <= 2 * WAVE) MOE_ROUTE(2);
+  else MOE_ROUTE(MOE_PER_LANE);
+#undef MOE_ROUTE
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -296,18 +302,32 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_up[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int k0 = 0; k0 < k_dim; k0 += 32) {
-    const bool in = k0 + 8 * g < k_dim;                       // K is a multiple of 8: a lane's eight are in or out
-    const bf16x8 wg = in ? *(const bf16x8*)(w_gate + k0) : zero;
-    bf16x8 wu = zero;
-    if (GLU && in) wu = *(const bf16x8*)(w_up + k0);
-    bf16x8 x[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) x[mt] = in ? *(const bf16x8*)(rows[mt] + k0) : zero;
+  // K in blocks of 64: lane (c, g) takes values 16 g .. 16 g + 15 of a block, 32 contiguous bytes of its row, for
+  // both operands alike (a sum over K does not mind the order), the first eight for one instruction and the second
+  // eight for the next; four lanes then cover a whole 128-byte line of a row.
+  for (int k0 = 0; k0 < k_dim; k0 += 64) {
+    const int at = k0 + 16 * g - 8 * g;                         // the row pointers already hold 8 g
+    const bool in0 = k0 + 16 * g < k_dim, in1 = k0 + 16 * g + 8 < k_dim;   // K is a multiple of 8
+    const bf16x8 wg0 = in0 ? *(const bf16x8*)(w_gate + at) : zero, wg1 = in1 ? *(const bf16x8*)(w_gate + at + 8) : zero;
+    bf16x8 wu0 = zero, wu1 = zero;
+    if (GLU) {
+      if (in0) wu0 = *(const bf16x8*)(w_up + at);
+      if (in1) wu1 = *(const bf16x8*)(w_up + at + 8);
+    }
+    bf16x8 x0[MT], x1[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg, x[mt], acc[mt], 0, 0, 0);
-      if (GLU) acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu, x[mt], acc_up[mt], 0, 0, 0);
+      x0[mt] = in0 ? *(const bf16x8*)(rows[mt] + at) : zero;
+      x1[mt] = in1 ? *(const bf16x8*)(rows[mt] + at + 8) : zero;
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg0, x0[mt], acc[mt], 0, 0, 0);
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg1, x1[mt], acc[mt], 0, 0, 0);
+      if (GLU) {
+        acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu0, x0[mt], acc_up[mt], 0, 0, 0);
+        acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu1, x1[mt], acc_up[mt], 0, 0, 0);
+      }
     }
   }
 #pragma unroll

@@ -75,7 +75,8 @@ _SIGNATURES = {
     "hyper": {"dryft_hyper_norm": [_P, _I, _I, _P, _I, _I, _L, _P, _P, _P, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "wkv": {"dryft_wkv_blend": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
             "dryft_wkv_decay": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
-            "dryft_wkv_steps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+            "dryft_wkv_steps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _I, _P, _P, _I,
+                                _P],
             "dryft_wkv_out": [_P, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "latent": {"dryft_rms_segments": [_P, _L, _I, _P, _P, _I, _P, _P, _I, _F, _I, _I, _P],
                "dryft_latent_rope_kv": [_P, _P, _P, _L, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
@@ -1393,8 +1394,8 @@ def wkv_blend(h, previous, mu, row_slot, row_seq, row_pos, seq_start, out) -> No
            "wkv_blend")
 
 
-def wkv_decay(low, up, bias, log_w) -> None:
-    """``log_w = -exp(tanh(low) @ up.T + bias)``: ``low`` float32 ``[rows, rank]``, ``up`` ``[n, rank]``."""
+def wkv_decay(low, up, bias, decay) -> None:
+    """``decay = exp(-exp(tanh(low) @ up.T + bias))``: ``low`` float32 ``[rows, rank]``, ``up`` ``[n, rank]``."""
     _gpu(low, "low", torch.float32)
     _gpu(up, "up")
     rows, rank = low.shape
@@ -1402,26 +1403,32 @@ def wkv_decay(low, up, bias, log_w) -> None:
     if not (low.is_contiguous() and up.is_contiguous() and up.shape == (n, rank)):
         raise KernelError(f"wkv_decay: low contiguous [rows, {rank}], up contiguous [n, {rank}], got {tuple(up.shape)}")
     _f32_vector(bias, "bias", n)
-    _gpu(log_w, "log_w", torch.float32)
-    if not (log_w.shape == (rows, n) and log_w.is_contiguous()):
-        raise KernelError("wkv_decay: log_w must be contiguous float32 [rows, n]")
-    _check(_fn("wkv", "dryft_wkv_decay")(_ptr(low), _ptr(up), _ptr(bias), _ptr(log_w), rows, n, rank,
+    _gpu(decay, "decay", torch.float32)
+    if not (decay.shape == (rows, n) and decay.is_contiguous()):
+        raise KernelError("wkv_decay: decay must be contiguous float32 [rows, n]")
+    _check(_fn("wkv", "dryft_wkv_decay")(_ptr(low), _ptr(up), _ptr(bias), _ptr(decay), rows, n, rank,
                                          _float_flag(up, "up"), _stream()), "wkv_decay")
 
 
-def wkv_steps(r, k, v, log_w, bonus, seq_slot, cu_rows, q_len, n_seqs: int, state, o_raw, h, previous, n_heads: int,
-              dim: int, write_state: bool) -> None:
+WKV_GROUP = 16          # tokens the recurrence's kernel takes at a time; segments are multiples of it
+
+
+def wkv_steps(r, k, v, decay, bonus, seq_slot, cu_rows, q_len, n_seqs: int, state, o_raw, h, previous, n_heads: int,
+              dim: int, write_state: bool, segments=None) -> None:
     """The recurrence over every sequence's rows in order, from ``state[slot]`` (float32 ``[slots, heads, dim, dim]``)
-    to the raw read-outs ``o_raw`` (float32 ``[rows, heads * dim]``); when ``write_state`` the state is written back
-    and ``previous[slot]`` receives the sequence's last row of ``h``."""
-    _gpu(r, "r")
-    rows = r.shape[0]
+    to the raw read-outs ``o_raw`` (float32 ``[rows, heads * dim]``); ``decay`` is float32, ``r``, ``k`` and ``v`` in the
+    activation dtype. When ``write_state`` the state is written back and ``previous[slot]`` receives the sequence's
+    last row of ``h``. ``segments = (rows per segment, prefix sums of segments over the sequences, their bound)``: long
+    sequences run as segments side by side, in three launches (every segment's summary from a zero state, the state
+    that enters each, every segment's outputs); the rows of sequences that sit out are then not written."""
+    _gpu(v, "v")
+    rows = v.shape[0]
     inner = n_heads * dim
     for name, t in (("r", r), ("k", k), ("v", v)):
-        _gpu(t, name, r.dtype)
+        _gpu(t, name, v.dtype)
         if not (t.shape == (rows, inner) and t.is_contiguous()):
             raise KernelError(f"wkv_steps: {name} must be contiguous [rows, {inner}]")
-    for name, t in (("log_w", log_w), ("o_raw", o_raw)):
+    for name, t in (("decay", decay), ("o_raw", o_raw)):
         _gpu(t, name, torch.float32)
         if not (t.shape == (rows, inner) and t.is_contiguous()):
             raise KernelError(f"wkv_steps: {name} must be contiguous float32 [rows, {inner}]")
@@ -1430,17 +1437,29 @@ def wkv_steps(r, k, v, log_w, bonus, seq_slot, cu_rows, q_len, n_seqs: int, stat
     _gpu(state, "state", torch.float32)
     if not (state.dim() == 4 and state.shape[1:] == (n_heads, dim, dim) and state.is_contiguous()):
         raise KernelError(f"wkv_steps: state must be contiguous float32 [slots, {n_heads}, {dim}, {dim}]")
-    _gpu(h, "h", r.dtype)
+    _gpu(h, "h", v.dtype)
     _gpu(previous, "previous", torch.float32)
     if not (h.dim() == 2 and h.shape[0] == rows and h.is_contiguous() and previous.dim() == 2 and
             previous.shape == (state.shape[0], h.shape[1]) and previous.is_contiguous()):
         raise KernelError("wkv_steps: h contiguous [rows, width], previous contiguous float32 [slots, width]")
     if not 0 < dim <= WKV_MAX_DIM:
         raise KernelError(f"wkv_steps: dim must lie in 1..{WKV_MAX_DIM}")
+    seg_cu = seg_state = seg_decay = None
+    seg_rows = max_segs = 0
+    if segments is not None:
+        seg_rows, seg_cu, max_segs = segments
+        _gpu(seg_cu, "segment prefix sums", torch.int32)
+        if not (seg_cu.numel() >= n_seqs + 1 and seg_rows > 0 and seg_rows % WKV_GROUP == 0 and write_state):
+            raise KernelError(f"wkv_steps: segments of a multiple of {WKV_GROUP} rows, prefix sums for every sequence, "
+                              "and a state that is written back")
+        if max_segs <= 0:
+            return
+        seg_state = torch.empty((max_segs, n_heads, dim, dim), dtype=torch.float32, device=v.device)
+        seg_decay = torch.empty((max_segs, n_heads, dim), dtype=torch.float32, device=v.device)
     _check(_fn("wkv", "dryft_wkv_steps")(
-        _ptr(r), _ptr(k), _ptr(v), _ptr(log_w), _ptr(bonus), _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs,
+        _ptr(r), _ptr(k), _ptr(v), _ptr(decay), _ptr(bonus), _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), n_seqs,
         _ptr(state), _ptr(o_raw), _ptr(h), _ptr(previous), h.shape[1], n_heads, dim, int(bool(write_state)),
-        _float_flag(r, "r"), _stream()), "wkv_steps")
+        _ptr(seg_cu), max_segs, seg_rows, _ptr(seg_state), _ptr(seg_decay), _float_flag(v, "v"), _stream()), "wkv_steps")
 
 
 def wkv_out(o_raw, gate, weight, out, n_heads: int, dim: int, eps: float) -> None:
