@@ -264,11 +264,18 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
 
 // The same on the matrix cores (bfloat16, K a multiple of 8, rows at 16-byte addresses). A wave owns 16 outputs (for
 // the gated unit 16 gate rows and the 16 up rows that go with them) and all 64 places of the tile: the weights are the
-// first operand of v_mfma_f32_16x16x32_bf16 (lane c + 16 g holds row c, values 8 g .. 8 g + 7 of a block of 32), the
-// operand rows the second, so accumulator entry i of lane (c, g) is output 4 g + i of place c. Operands go straight
-// from memory into that layout, 16 bytes a lane; every weight is read by one wave of the workgroup.
+// first operand of v_mfma_f32_16x16x32_bf16, the operand rows the second, so accumulator entry i of lane (c, g) is
+// output 4 g + i of place c. K goes in blocks of 64: lane (c, g) takes values 16 g .. 16 g + 15 of a block, 32
+// contiguous bytes of its row, for both operands alike (a sum over K does not mind the order), the first eight for
+// one instruction and the second eight for the next; four lanes then cover a whole 128-byte line of a row. Weights
+// go straight from memory into that layout and every weight is read by one wave of the workgroup; the 64 operand
+// rows, which all four waves need, go through LDS (gathered once per workgroup, two buffers, the next block of K on
+// its way while this one is multiplied; rows 144 bytes apart so that 16 rows' 16-byte pieces fall into different
+// banks).
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define MOE_X_STRIDE 72      // bf16 elements between two operand rows in LDS: 64 values and 16 bytes
 
 template <typename O, bool GLU>
 __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __restrict__ a, int64_t a_stride,
@@ -280,56 +287,63 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
                                                                const int* __restrict__ n_tiles, O* __restrict__ out,
                                                                int top, int n_out, int k_dim, float limit, float alpha) {
   constexpr int MT = MOE_TILE / 16;
+  __shared__ __attribute__((aligned(16))) bf16_t sx[2][MOE_TILE * MOE_X_STRIDE];
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
   const int n0 = (blockIdx.y * 4 + wave) * 16;
-  if (n0 >= n_out) return;
+  const bool works = n0 < n_out;                              // a wave without outputs still helps to bring rows in
   const int expert = tile_expert[tile], start = tile_start[tile], count = tile_rows[tile];
   const int w_rows = GLU ? 2 * n_out : n_out;
   const bf16_t* we = w + (int64_t)expert * w_rows * k_dim;
   const int n_mine = min(n0 + c, n_out - 1);                  // rows beyond the last are read from it and never stored
-  const bf16_t* w_gate = we + (int64_t)n_mine * k_dim + 8 * g;
-  const bf16_t* w_up = we + ((int64_t)n_out + n_mine) * k_dim + 8 * g;
-  const bf16_t* rows[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int place = start + min(16 * mt + c, count - 1);    // places beyond the tile's: its last one, never stored
-    const int row = top > 0 ? sorted_pair[place] / top : place;
-    rows[mt] = a + (int64_t)row * a_stride + 8 * g;
-  }
+  const bf16_t* w_gate = we + (int64_t)n_mine * k_dim + 16 * g;
+  const bf16_t* w_up = we + ((int64_t)n_out + n_mine) * k_dim + 16 * g;
+  // staging: thread (row = tid / 4, piece = tid % 4) brings 32 bytes of its row per block of K
+  const int s_row = threadIdx.x / 4, s_piece = threadIdx.x % 4;
+  const int s_place = start + min(s_row, count - 1);          // places beyond the tile's: its last one, never stored
+  const bf16_t* s_src = a + (int64_t)(top > 0 ? sorted_pair[s_place] / top : s_place) * a_stride + 16 * s_piece;
+  const int s_at = s_row * MOE_X_STRIDE + 16 * s_piece;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  bf16x8 p0, p1;
+  auto fetch = [&](int k0) {
+    p0 = k0 + 16 * s_piece < k_dim ? *(const bf16x8*)(s_src + k0) : zero;          // K is a multiple of 8
+    p1 = k0 + 16 * s_piece + 8 < k_dim ? *(const bf16x8*)(s_src + k0 + 8) : zero;
+  };
   f32x4 acc[MT], acc_up[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = acc_up[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  // K in blocks of 64: lane (c, g) takes values 16 g .. 16 g + 15 of a block, 32 contiguous bytes of its row, for
-  // both operands alike (a sum over K does not mind the order), the first eight for one instruction and the second
-  // eight for the next; four lanes then cover a whole 128-byte line of a row.
-  for (int k0 = 0; k0 < k_dim; k0 += 64) {
-    const int at = k0 + 16 * g - 8 * g;                         // the row pointers already hold 8 g
-    const bool in0 = k0 + 16 * g < k_dim, in1 = k0 + 16 * g + 8 < k_dim;   // K is a multiple of 8
-    const bf16x8 wg0 = in0 ? *(const bf16x8*)(w_gate + at) : zero, wg1 = in1 ? *(const bf16x8*)(w_gate + at + 8) : zero;
-    bf16x8 wu0 = zero, wu1 = zero;
-    if (GLU) {
-      if (in0) wu0 = *(const bf16x8*)(w_up + at);
-      if (in1) wu1 = *(const bf16x8*)(w_up + at + 8);
+  fetch(0);
+  int buf = 0;
+  for (int k0 = 0; k0 < k_dim; k0 += 64, buf ^= 1) {
+    *(bf16x8*)(sx[buf] + s_at) = p0;
+    *(bf16x8*)(sx[buf] + s_at + 8) = p1;
+    if (k0 + 64 < k_dim) fetch(k0 + 64);
+    bf16x8 wg0 = zero, wg1 = zero, wu0 = zero, wu1 = zero;
+    if (works) {
+      const bool in0 = k0 + 16 * g < k_dim, in1 = k0 + 16 * g + 8 < k_dim;
+      if (in0) wg0 = *(const bf16x8*)(w_gate + k0);
+      if (in1) wg1 = *(const bf16x8*)(w_gate + k0 + 8);
+      if (GLU && in0) wu0 = *(const bf16x8*)(w_up + k0);
+      if (GLU && in1) wu1 = *(const bf16x8*)(w_up + k0 + 8);
     }
-    bf16x8 x0[MT], x1[MT];
+    __syncthreads();               // this buffer is whole; the other one was last read before the barrier before
+    if (works) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      x0[mt] = in0 ? *(const bf16x8*)(rows[mt] + at) : zero;
-      x1[mt] = in1 ? *(const bf16x8*)(rows[mt] + at + 8) : zero;
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg0, x0[mt], acc[mt], 0, 0, 0);
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg1, x1[mt], acc[mt], 0, 0, 0);
-      if (GLU) {
-        acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu0, x0[mt], acc_up[mt], 0, 0, 0);
-        acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu1, x1[mt], acc_up[mt], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        if (16 * mt >= count) break;                            // a tile of few places (decoding) skips the empty rows
+        const bf16_t* xr = sx[buf] + (16 * mt + c) * MOE_X_STRIDE + 16 * g;
+        const bf16x8 x0 = *(const bf16x8*)xr, x1 = *(const bf16x8*)(xr + 8);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg0, x0, acc[mt], 0, 0, 0);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg1, x1, acc[mt], 0, 0, 0);
+        if (GLU) {
+          acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu0, x0, acc_up[mt], 0, 0, 0);
+          acc_up[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu1, x1, acc_up[mt], 0, 0, 0);
+        }
       }
     }
   }
+  if (!works) return;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = 16 * mt + c;
@@ -392,7 +406,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           int shared_col, T* __restrict__ out, int top, int width) {
   const int64_t row = blockIdx.x;
   const float gate = shared ? 1.f / (1.f + expf(-logits[row * logit_stride + shared_col])) : 0.f;
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k)
       acc += weights[row * top + k] * y[(int64_t)place_of[row * top + k] * width + c];
@@ -405,11 +419,12 @@ DRYFT_API int dryft_moe_combine(const float* y, const int* place_of, const float
                                 const float* logits, int64_t logit_stride, int shared_col, void* out, int rows, int top,
                                 int width, int is_f32, hipStream_t stream) {
   if (rows <= 0) return 0;
+  const dim3 grid(rows, rows <= 64 ? (width + 255) / 256 : 1);       // few rows: a workgroup per 256 columns
   if (is_f32)
-    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(rows), dim3(256), 0, stream, y, place_of, weights,
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, y, place_of, weights,
                        (const float*)shared, logits, logit_stride, shared_col, (float*)out, top, width);
   else
-    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(rows), dim3(256), 0, stream, y, place_of, weights,
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, dim3(256), 0, stream, y, place_of, weights,
                        (const bf16_t*)shared, logits, logit_stride, shared_col, (bf16_t*)out, top, width);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void wkv_decay_kernel(const float* __restrict_
     t_low[i] = row < rows ? tanhf(low[row * rank + i % rank]) : 0.f;
   }
   __syncthreads();
-  for (int n = threadIdx.x; n < n_out; n += blockDim.x) {
+  for (int n = blockIdx.y * blockDim.x + threadIdx.x; n < n_out; n += gridDim.y * blockDim.x) {
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = 0.f;
@@ -92,7 +92,7 @@ DRYFT_API int dryft_wkv_decay(const float* low, const void* up, const float* bia
   if (rank <= 0 || rank > 2048) return -1;
   if (rows >= 64) {
     const size_t lds = (size_t)8 * rank * sizeof(float);
-    dim3 grid((rows + 7) / 8);
+    dim3 grid((rows + 7) / 8, 1);
     if (up_is_f32)
       hipLaunchKernelGGL((wkv_decay_kernel<float, 8>), grid, dim3(256), lds, stream, low, (const float*)up, bias, decay,
                          rows, n_out, rank);
@@ -101,11 +101,12 @@ DRYFT_API int dryft_wkv_decay(const float* low, const void* up, const float* bia
                          rows, n_out, rank);
   } else {
     const size_t lds = (size_t)rank * sizeof(float);
+    dim3 grid(rows, (n_out + 255) / 256);          // few rows: a workgroup per 256 outputs, so that the chip has work
     if (up_is_f32)
-      hipLaunchKernelGGL((wkv_decay_kernel<float, 1>), dim3(rows), dim3(256), lds, stream, low, (const float*)up, bias,
+      hipLaunchKernelGGL((wkv_decay_kernel<float, 1>), grid, dim3(256), lds, stream, low, (const float*)up, bias,
                          decay, rows, n_out, rank);
     else
-      hipLaunchKernelGGL((wkv_decay_kernel<bf16_t, 1>), dim3(rows), dim3(256), lds, stream, low, (const bf16_t*)up, bias,
+      hipLaunchKernelGGL((wkv_decay_kernel<bf16_t, 1>), grid, dim3(256), lds, stream, low, (const bf16_t*)up, bias,
                          decay, rows, n_out, rank);
   }
   return DRYFT_LAUNCH_CHECK();
