@@ -477,6 +477,21 @@ def test_greedy_generation_through_the_entry_point(models, name, dtype):
     assert engine.generate_all(prompts, 8) == first
 
 
+def test_a_long_prompt_in_a_captured_step(models):
+    """A prompt long enough for the wkv mixer to cut it into segments, started in a captured step beside a short one
+    and a sequence that sits out to fill the step: the same tokens as without captured steps (float32, where the two
+    differ by rounding far below any gap between logits)."""
+    model = models["A"]
+    prompts = [model.tokens(150, seed=4), model.tokens(3, seed=5)]
+    got = {}
+    for use_graph in (True, False):
+        engine = model.engine("float32", max_batch=4, max_len=192, max_tokens=64 * 12, use_graph=use_graph)
+        got[use_graph] = engine.generate_all(prompts, 6)
+    assert got[True] == got[False]
+    want, _ = plain_greedy(model, prompts[0], 6)
+    assert got[False][0] == want
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_program(models, dtype, tmp_path):
     model = models["C"]
