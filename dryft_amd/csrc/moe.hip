@@ -363,14 +363,90 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
   }
 }
 
+// For steps of few rows (decoding), where a tile holds at most 16 places: no LDS and no barrier. A wave walks K for
+// its 16 outputs with the operand rows straight from memory (they are few and stay in the vector cache) and four
+// blocks of K in flight, so that the weights, which are all the step reads, stream. Tiles of more places are walked
+// 16 places at a time.
+template <typename O, bool GLU>
+__global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __restrict__ a, int64_t a_stride,
+                                                              const bf16_t* __restrict__ w,
+                                                              const int* __restrict__ sorted_pair,
+                                                              const int* __restrict__ tile_expert,
+                                                              const int* __restrict__ tile_start,
+                                                              const int* __restrict__ tile_rows,
+                                                              const int* __restrict__ n_tiles, O* __restrict__ out,
+                                                              int top, int n_out, int k_dim, float limit, float alpha) {
+  const int tile = blockIdx.x;
+  if (tile >= *n_tiles) return;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
+  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  if (n0 >= n_out) return;
+  const int expert = tile_expert[tile], start = tile_start[tile], count = tile_rows[tile];
+  const int w_rows = GLU ? 2 * n_out : n_out;
+  const bf16_t* we = w + (int64_t)expert * w_rows * k_dim;
+  const int n_mine = min(n0 + c, n_out - 1);
+  const bf16_t* w_gate = we + (int64_t)n_mine * k_dim + 16 * g;
+  const bf16_t* w_up = we + ((int64_t)n_out + n_mine) * k_dim + 16 * g;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int m0 = 0; m0 < count; m0 += 16) {
+    const int place = start + min(m0 + c, count - 1);
+    const bf16_t* x = a + (int64_t)(top > 0 ? sorted_pair[place] / top : place) * a_stride + 16 * g;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < k_dim; k0 += 256) {
+      bf16x8 wg[8], wu[8], xv[8];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + 64 * u;
+        const bool in0 = k + 16 * g < k_dim, in1 = k + 16 * g + 8 < k_dim;     // K is a multiple of 8
+        wg[2 * u] = in0 ? *(const bf16x8*)(w_gate + k) : zero;
+        wg[2 * u + 1] = in1 ? *(const bf16x8*)(w_gate + k + 8) : zero;
+        wu[2 * u] = (GLU && in0) ? *(const bf16x8*)(w_up + k) : zero;
+        wu[2 * u + 1] = (GLU && in1) ? *(const bf16x8*)(w_up + k + 8) : zero;
+        xv[2 * u] = in0 ? *(const bf16x8*)(x + k) : zero;
+        xv[2 * u + 1] = in1 ? *(const bf16x8*)(x + k + 8) : zero;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wg[u], xv[u], acc, 0, 0, 0);
+        if (GLU) acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wu[u], xv[u], acc_up, 0, 0, 0);
+      }
+    }
+    const int m = m0 + c;
+    if (m >= count) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g + i;
+      if (n >= n_out) continue;
+      float v = acc[i];
+      if (GLU) {
+        const float gv = fminf(rounded_as<bf16_t>(v), limit);
+        const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[i]), -limit), limit);
+        v = gv / (1.f + expf(-alpha * gv)) * (uv + 1.f);
+      }
+      store_from_float(out + (int64_t)(start + m) * n_out + n, v);
+    }
+  }
+}
+
 DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, const int* sorted_pair,
                                 const int* tile_expert, const int* tile_start, const int* tile_rows, const int* n_tiles,
                                 int max_tiles, void* out, int out_is_f32, int top, int n_out, int k_dim, int glu,
-                                float limit, float alpha, int is_f32, hipStream_t stream) {
+                                float limit, float alpha, int most_places, int is_f32, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || k_dim <= 0 || (glu && out_is_f32 && !is_f32)) return -1;
   dim3 grid(max_tiles, (n_out + MOE_TN - 1) / MOE_TN), block(256);
   if (!is_f32 && k_dim % 8 == 0 && a_stride % 8 == 0 && (((uintptr_t)a | (uintptr_t)w) & 15) == 0) {
+    if (most_places <= 16) {           // no expert can get more places than that: the kernel without LDS and barriers
+#define MOE_FEW(O, G)                                                                                             \
+  hipLaunchKernelGGL((moe_product_few_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,           \
+                     (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
+                     k_dim, limit, alpha)
+      if (glu) MOE_FEW(bf16_t, true);
+      else if (out_is_f32) MOE_FEW(float, false);
+      else MOE_FEW(bf16_t, false);
+#undef MOE_FEW
+      return DRYFT_LAUNCH_CHECK();
+    }
 #define MOE_MFMA(O, G)                                                                                            \
   hipLaunchKernelGGL((moe_product_mfma_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,          \
                      (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \

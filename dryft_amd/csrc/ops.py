@@ -84,7 +84,7 @@ _SIGNATURES = {
                "dryft_head_gate": [_P, _P, _L, _I, _P, _I, _I, _I, _I, _I, _P]},
     "moe": {"dryft_moe_route": [_P, _L, _P, _I, _I, _I, _I, _F, _P, _P, _I, _P],
             "dryft_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
-            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I, _P],
+            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
             "dryft_moe_combine": [_P, _P, _P, _P, _P, _L, _I, _P, _I, _I, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _I, _P, _P, _P]},
@@ -1584,10 +1584,12 @@ def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale:
 
 class MoePlan:
     """Where each (row, expert) pair of a step sits once the pairs are sorted by expert, and the tiles of the sorted
-    run, all on the device."""
+    run, all on the device. ``most_places``: what the host knows no expert's run to exceed (a row chooses an expert
+    once, so the step's rows)."""
 
-    def __init__(self, n_pairs: int, n_experts: int, device):
+    def __init__(self, n_pairs: int, n_experts: int, device, most_places: int | None = None):
         self.n_pairs = n_pairs
+        self.most_places = n_pairs if most_places is None else int(most_places)
         self.max_tiles = n_pairs // MOE_TILE + min(n_experts, n_pairs)
         i32 = dict(dtype=torch.int32, device=device)
         self.sorted_pair = torch.empty(n_pairs, **i32)
@@ -1600,7 +1602,7 @@ def moe_plan(chosen, n_experts: int) -> MoePlan:
     _gpu(chosen, "chosen", torch.int32)
     if not chosen.is_contiguous():
         raise KernelError("moe_plan: chosen must be contiguous")
-    plan = MoePlan(chosen.numel(), n_experts, chosen.device)
+    plan = MoePlan(chosen.numel(), n_experts, chosen.device, most_places=chosen.shape[0] if chosen.dim() == 2 else None)
     _check(_fn("moe", "dryft_moe_plan")(_ptr(chosen), plan.n_pairs, n_experts, _ptr(plan.sorted_pair), _ptr(plan.place_of),
                                         _ptr(plan.tiles[0]), _ptr(plan.tiles[1]), _ptr(plan.tiles[2]), _ptr(plan.n_tiles),
                                         plan.max_tiles, _stream()), "moe_plan")
@@ -1631,7 +1633,8 @@ def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple[float, float] | 
     _check(_fn("moe", "dryft_moe_product")(
         _ptr(a), a.stride(0), _ptr(w), _ptr(plan.sorted_pair), _ptr(plan.tiles[0]), _ptr(plan.tiles[1]),
         _ptr(plan.tiles[2]), _ptr(plan.n_tiles), plan.max_tiles, _ptr(out), 1 if out.dtype == torch.float32 else 0,
-        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), _float_flag(a, "a"), _stream()), "moe_products")
+        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), plan.most_places, _float_flag(a, "a"), _stream()),
+        "moe_products")
 
 
 def moe_combine(y, plan: MoePlan, weights, shared, logits, shared_col: int, out) -> None:
